@@ -21,7 +21,6 @@
 //     (amdgpu_num_vgpr) for addresses and the drain's temporaries; every register above is named by hand in inline asm.
 //   * barriers sit one step BEHIND the last fragment read of the region they release, so no LDS latency is exposed in front
 //     of them, and fragments stay valid across a tile boundary (nothing is re-read).
-// Audit after every edit (tools/README.md): no compiler-generated v_accvgpr_* and no scratch in the -S output.
 #include <stdlib.h>
 
 #include <type_traits>

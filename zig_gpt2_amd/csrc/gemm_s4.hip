@@ -118,8 +118,7 @@ __device__ __forceinline__ void read_frag_b(bf16x8& f, const unsigned (&b_addr)[
 // MFMAs below and read / zeroed only by the inline-asm moves of the epilogue.  Left to the register allocator, a change in
 // the epilogue's register pressure made it park accumulators in VGPRs and shuffle them with v_accvgpr_mov inside the K loop
 // (dependent on the MFMAs: +14k cycles per launch).  Every statement that touches them names all of them as clobbered, so
-// the compiler keeps nothing of its own there across any of them; what remains to audit after an edit is that no
-// compiler-generated v_accvgpr_* names a0..a191 (tools/README: grep recipe).  Hazards are ours too: MFMA result ->
+// the compiler keeps nothing of its own there across any of them.  Hazards are ours too: MFMA result ->
 // v_accvgpr_read needs the pipeline drained (s_nop in acc_settle), v_accvgpr_write -> MFMA source C two wait states.
 #define ZG_ACC_CLOBBERS "a0","a1","a2","a3","a4","a5","a6","a7","a8","a9","a10","a11","a12","a13","a14","a15","a16","a17","a18","a19","a20","a21","a22","a23","a24","a25","a26","a27","a28","a29","a30","a31","a32","a33","a34","a35","a36","a37","a38","a39","a40","a41","a42","a43","a44","a45","a46","a47","a48","a49","a50","a51","a52","a53","a54","a55","a56","a57","a58","a59","a60","a61","a62","a63","a64","a65","a66","a67","a68","a69","a70","a71","a72","a73","a74","a75","a76","a77","a78","a79","a80","a81","a82","a83","a84","a85","a86","a87","a88","a89","a90","a91","a92","a93","a94","a95","a96","a97","a98","a99","a100","a101","a102","a103","a104","a105","a106","a107","a108","a109","a110","a111","a112","a113","a114","a115","a116","a117","a118","a119","a120","a121","a122","a123","a124","a125","a126","a127","a128","a129","a130","a131","a132","a133","a134","a135","a136","a137","a138","a139","a140","a141","a142","a143","a144","a145","a146","a147","a148","a149","a150","a151","a152","a153","a154","a155","a156","a157","a158","a159","a160","a161","a162","a163","a164","a165","a166","a167","a168","a169","a170","a171","a172","a173","a174","a175","a176","a177","a178","a179","a180","a181","a182","a183","a184","a185","a186","a187","a188","a189","a190","a191"
 template <int BASE>
