@@ -337,6 +337,90 @@ int zg_gpt_generate_enqueue_many(zg_gpt* const* handles, size_t n_handles, const
                                  const size_t* prompt_lens, size_t n_steps);
 int zg_gpt_generate_fetch_many(zg_gpt* const* handles, size_t n_handles, size_t n_steps, size_t* out_tokens, size_t out_len);
 
+/* ------------------------------------------------------------------ layered-model tier ------
+ * Decoder stacks described by DATA (no reference counterpart: src/main.zig hard-codes the GPT-2 block): every layer names its
+ * token mixer and its feed-forward with their sizes, a span of layers may run several times in a row with the same weights,
+ * and sequences are served from state slots — a paged cache of attention latents, the recurrent state of the linear-recurrence
+ * layers, the previous token's row of every layer's token shift — that are opened, stepped with any number of tokens at a time
+ * (prompt portions and single decoded tokens alike, several sequences in one step), and closed again.  Which checkpoint
+ * architecture maps to which layer list is the host program's business (zig_gpt2_amd/models.py, zig_gpt2_amd/lm.py).
+ *
+ * A layer computes   x += norm1b(mixer(shift(norm1(x))));   x += norm2b(ff(norm2(x)))
+ * with RMS norms whose stored weight is an offset from one, and shift(h)_t = h_t + (h_(t-1) - h_t) * mu.
+ * Norms, softmax, router, gates, recurrent state, positions and the residual are fp32; matrix products take bf16 operands with
+ * fp32 accumulation, or true fp32 products under ZG_LM_F32.  Weights are stored bf16. */
+enum {
+    ZG_LM_MIX_HGRN2 = 1,            /* gated linear recurrence: S = diag(f) S + (1 - f) v^T, o = S^T q, f bounded from below */
+    ZG_LM_MIX_LATENT_ATTENTION = 2  /* causal softmax attention whose keys and values are up-projections of a cached latent, plus
+                                       one rotary key part shared by the heads; queries through a latent of their own */
+};
+enum { ZG_LM_FF_NONE = 0, ZG_LM_FF_DENSE = 1 /* down(relu(up h)^2) */, ZG_LM_FF_MOE = 2 /* top-k of `experts` gated units */ };
+typedef struct {
+    int mixer;                    /* ZG_LM_MIX_* */
+    int heads, dim, vdim;         /* both mixers: heads, key (unrotated) channels and value channels per head */
+    int rot_dim, kv_rank, q_rank; /* latent attention: rotated channels per head, latent sizes of keys/values and of queries */
+    float scale;                  /* latent attention: factor of the scores */
+    int rot_dims;                 /* rotary: how many of the rot_dim channels are rotated (interleaved pairs) */
+    float rot_base;
+    int rot_scaled;               /* != 0: YaRN blend of the frequencies with the four constants below */
+    float rot_factor, rot_original, rot_fast, rot_slow;
+    int ff;                       /* ZG_LM_FF_* */
+    int ff_width;                 /* hidden width of the dense feed-forward, or of ONE expert */
+    int experts, top;
+} zg_lm_layer;
+enum { ZG_LM_F32 = 1 << 0 /* true 32-bit products everywhere */ };
+typedef struct {
+    size_t vocab, width, n_layers;
+    const zg_lm_layer* layers;
+    int loop_start, loop_stop, loop_times; /* layers [start, stop) run `times` times in a row, every pass with a state of its own; times <= 1: no loop */
+    float norm_eps;
+    size_t max_tokens;      /* tokens that all open sequences may hold together (sizes the latent cache) */
+    size_t max_seqs;        /* state slots */
+    size_t max_step_tokens; /* rows of one pass; a longer step is cut into portions (0: 2048) */
+    size_t page_tokens;     /* tokens per cache page (0: 64) */
+    unsigned flags;         /* ZG_LM_* */
+} zg_lm_config;
+typedef struct zg_lm zg_lm;
+/* One arena for weights, state and scratch; the handle owns a stream on `device`.  Needs no zg_init. */
+int zg_lm_create(zg_lm** out, const zg_lm_config* config, int device);
+int zg_lm_destroy(zg_lm* g);
+/* Weights by checkpoint name: `embed`, `head`, `final.norm`, and per layer i `l<i>.norm1|norm1b|norm2|norm2b|shift`,
+ * `l<i>.mix.*` (hgrn2: q f f.b lower v norm o; latent attention: dq dq.norm uq dkv dkv.norm uk uv o) and `l<i>.mlp.*`
+ * (dense: up down; experts: e<j>.gate e<j>.up e<j>.down router correction).  data: fp32 on the host, `len` elements, matrices
+ * [out][in] row-major; matrices are stored bf16 (round to nearest even).  ZG_ERR_ARG for a name the configuration does not have. */
+int zg_lm_load_tensor(zg_lm* g, const char* name, const float* data, size_t len);
+/* How many tensors of the configuration have not been loaded; names_out (may be NULL) receives them, space separated. */
+int zg_lm_missing_tensors(zg_lm* g, size_t* count, char* names_out, size_t names_cap);
+/* Every tensor ~ N(0, std^2) (norm offsets, shift, lower bounds in [0, 1)) from a counter PRNG, filled on the device: benchmarks. */
+int zg_lm_init_random(zg_lm* g, uint64_t seed, float std);
+/* State slots.  open: a free slot with zeroed state; close: its pages and the slot return to the pool. */
+int zg_lm_seq_open(zg_lm* g, int* seq_out);
+int zg_lm_seq_close(zg_lm* g, int seq);
+int zg_lm_seq_len(zg_lm* g, int seq, size_t* len_out);
+int zg_lm_free_tokens(zg_lm* g, size_t* tokens_out); /* tokens the free pages can still take */
+/* One step: every entry appends n_tokens tokens to its sequence; `want` lists the places among them (0-based, any order)
+ * whose logits are asked for.  logits_out (host, fp32) receives [sum of n_want][vocab] rows in entry order, then want order.
+ * Portions may be cut anywhere; the logits of a position do not depend on the cut or on the other entries beyond rounding. */
+typedef struct {
+    int seq;
+    const int32_t* tokens;
+    size_t n_tokens;
+    const int32_t* want;
+    size_t n_want;
+} zg_lm_entry;
+int zg_lm_step(zg_lm* g, const zg_lm_entry* entries, size_t n_entries, float* logits_out, size_t logits_len);
+/* Generation through the same step: prompts [n_prompts][prompt_stride] with prompt_lens tokens each are fed in portions, then
+ * all sequences decode in one batch per step; temp == 0: greedy (first maximum), else softmax(logits / temp) sampled with the
+ * library's counter PRNG of (seed, position, sequence) as zg_gpt_sample does.  out_tokens [n_prompts][n_new].  The sequences are
+ * opened and closed by the call. */
+int zg_lm_generate(zg_lm* g, const int32_t* prompts, size_t prompt_stride, const size_t* prompt_lens, size_t n_prompts, size_t n_new, float temp,
+                   uint64_t seed, int32_t* out_tokens, size_t out_len);
+/* Test hook: while set, every step copies the residual stream behind each layer pass into trace_out (host,
+ * [passes][rows of the step][width]; steps of at most max_step_tokens rows).  NULL switches it off. */
+int zg_lm_set_trace(zg_lm* g, float* trace_out, size_t trace_floats);
+/* Measurement: device time (ms) of the last zg_lm_step / of the decode steps of the last zg_lm_generate (events on the handle's stream). */
+int zg_lm_last_ms(zg_lm* g, float* step_ms, float* decode_ms_per_step);
+
 /* ------------------------------------------------------------------ measurement helpers ---- */
 
 /* Replay one kernel class of the decode step (layer 0; classes numbered as in

@@ -12,7 +12,10 @@ CSRC = os.path.join(_HERE, "csrc")
 SO_PATH = os.environ.get("ZGPT2_LIB") or os.path.join(_HERE, "lib", "libzgpt2_hip.so")  # ZGPT2_LIB: diagnostic builds
 HEADER = os.path.join(os.path.dirname(_HERE), "include", "zgpt2.h")
 
+LM_SO_PATH = os.path.join(_HERE, "lib", "libzgpt2_lm.so")  # the layered-model tier alone (make lm)
+
 _lib = None
+_lm_lib = None
 
 f32p = C.POINTER(C.c_float)
 szp = C.POINTER(C.c_size_t)
@@ -37,6 +40,52 @@ class GptOptions(C.Structure):
 
     _fields_ = [("share_weights_with", vp), ("own_stream", C.c_int), ("stream_priority", C.c_int)]
 
+
+class LmLayer(C.Structure):
+    """zg_lm_layer of include/zgpt2.h."""
+
+    _fields_ = [("mixer", C.c_int), ("heads", C.c_int), ("dim", C.c_int), ("vdim", C.c_int), ("rot_dim", C.c_int), ("kv_rank", C.c_int),
+                ("q_rank", C.c_int), ("scale", C.c_float), ("rot_dims", C.c_int), ("rot_base", C.c_float), ("rot_scaled", C.c_int),
+                ("rot_factor", C.c_float), ("rot_original", C.c_float), ("rot_fast", C.c_float), ("rot_slow", C.c_float), ("ff", C.c_int),
+                ("ff_width", C.c_int), ("experts", C.c_int), ("top", C.c_int)]
+
+
+class LmConfig(C.Structure):
+    """zg_lm_config of include/zgpt2.h."""
+
+    _fields_ = [("vocab", sz), ("width", sz), ("n_layers", sz), ("layers", C.POINTER(LmLayer)), ("loop_start", C.c_int), ("loop_stop", C.c_int),
+                ("loop_times", C.c_int), ("norm_eps", C.c_float), ("max_tokens", sz), ("max_seqs", sz), ("max_step_tokens", sz),
+                ("page_tokens", sz), ("flags", C.c_uint)]
+
+
+class LmEntry(C.Structure):
+    """zg_lm_entry of include/zgpt2.h."""
+
+    _fields_ = [("seq", C.c_int), ("tokens", vp), ("n_tokens", sz), ("want", vp), ("n_want", sz)]
+
+
+LM_MIX_HGRN2, LM_MIX_LATENT_ATTENTION = 1, 2
+LM_FF_NONE, LM_FF_DENSE, LM_FF_MOE = 0, 1, 2
+LM_F32 = 1
+
+# the layered-model tier (present in both libraries)
+LM_SIGNATURES = {
+    "zg_last_error": (C.c_char_p, []),
+    "zg_debug_last_kernel": (C.c_int, [C.c_char_p, sz]),
+    "zg_lm_create": (C.c_int, [C.POINTER(vp), C.POINTER(LmConfig), C.c_int]),
+    "zg_lm_destroy": (C.c_int, [vp]),
+    "zg_lm_load_tensor": (C.c_int, [vp, C.c_char_p, vp, sz]),
+    "zg_lm_missing_tensors": (C.c_int, [vp, szp, C.c_char_p, sz]),
+    "zg_lm_init_random": (C.c_int, [vp, C.c_uint64, C.c_float]),
+    "zg_lm_seq_open": (C.c_int, [vp, C.POINTER(C.c_int)]),
+    "zg_lm_seq_close": (C.c_int, [vp, C.c_int]),
+    "zg_lm_seq_len": (C.c_int, [vp, C.c_int, szp]),
+    "zg_lm_free_tokens": (C.c_int, [vp, szp]),
+    "zg_lm_step": (C.c_int, [vp, C.POINTER(LmEntry), sz, vp, sz]),
+    "zg_lm_generate": (C.c_int, [vp, vp, sz, vp, sz, sz, C.c_float, C.c_uint64, vp, sz]),
+    "zg_lm_set_trace": (C.c_int, [vp, vp, sz]),
+    "zg_lm_last_ms": (C.c_int, [vp, f32p, f32p]),
+}
 
 # name -> (restype, argtypes); every symbol include/zgpt2.h declares
 SIGNATURES = {
@@ -101,6 +150,7 @@ SIGNATURES = {
     "zg_bpe_encode": (C.c_int, [vp, C.c_char_p, sz, vp, sz, szp]),
     "zg_bpe_decode": (C.c_int, [vp, vp, sz, vp, sz, szp]),
 }
+SIGNATURES.update(LM_SIGNATURES)
 
 # flags / slots of include/zgpt2.h
 GPT_WEIGHTS_BF16, GPT_WEIGHTS_F32, GPT_NO_GRAPH, GPT_KV_F16, GPT_NO_PREFILL, GPT_PREFILL_2PLANE, GPT_NO_PREFETCH = 0, 1, 2, 4, 8, 16, 32
@@ -149,9 +199,48 @@ def load():
     return lib
 
 
+def build_lm():
+    """hipcc build of the layered-model tier alone into lib/libzgpt2_lm.so (`make lm`: a handful of files)."""
+    subprocess.check_call(["make", "-C", CSRC, "-j16", "lm"], stdout=subprocess.DEVNULL)
+    if not os.path.exists(LM_SO_PATH):
+        raise RuntimeError(f"build did not produce {LM_SO_PATH}")
+    return LM_SO_PATH
+
+
+def load_lm(build_if_missing=False):
+    """The library that holds the layered-model tier (zg_lm_*): the full library when it is built, else the tier's own small
+    library; with build_if_missing a fresh checkout compiles the latter (and only that) first.  No CPU fallback."""
+    global _lm_lib
+    if _lm_lib is not None:
+        return _lm_lib
+    if _lib is not None or os.path.exists(SO_PATH):
+        _lm_lib = load()
+        return _lm_lib
+    if not os.path.exists(LM_SO_PATH):
+        if not build_if_missing:
+            raise RuntimeError(f"{LM_SO_PATH} is missing: build it with `make -C {CSRC} lm` (or the whole library)")
+        build_lm()
+    try:
+        import torch  # noqa: F401  (one HIP runtime per process: see load())
+    except ImportError:
+        pass
+    lib = C.CDLL(LM_SO_PATH)
+    for name, (res, args) in LM_SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    _lm_lib = lib
+    return lib
+
+
 def check(code):
     if code != 0:
         raise ZgError(code, load().zg_last_error().decode(errors="replace"))
+
+
+def check_lm(code):
+    if code != 0:
+        raise ZgError(code, load_lm().zg_last_error().decode(errors="replace"))
 
 
 def ptr(a):

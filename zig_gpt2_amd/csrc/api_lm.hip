@@ -1,0 +1,907 @@
+// api_lm.hip — the layered-model tier of the C ABI (include/zgpt2.h, zg_lm_*): decoder stacks described by data, served from
+// state slots.  This file is the host side: the arena and the tensor table, the slot / page manager, the step function that
+// turns a ragged batch of entries into portions of rows and launches the kernels of lm_linear.hip / lm_mix.hip / lm_moe.hip
+// for every layer pass, and generation on top of the same step.
+//
+// Arena (one hipMalloc):
+//   [ weights: bf16 matrices [out][in], fp32 vectors; fused where one product serves several projections:
+//       hgrn2  qfv = q | f | v rows;   latent attention  dqkv = dq | dkv rows, uk kept TRANSPOSED per head ([H][kv_rank][dim]) so that
+//       the query can be carried into the latent space by an ordinary [out][in] product;   experts  gu = gate | up rows per expert ]
+//   [ state: token-shift rows [slot][pass][W] | recurrent states [slot][hgrn passes][H D V] | page table [slot][pages] |
+//       latent cache per attention pass [page][token][kv_rank + rot_dim] ]          all fp32
+//   [ scratch of one portion (max_step_tokens rows) | step metadata | logits ]
+//
+// Latent attention runs in its absorbed form in prompts and in decoding alike: score_j = (W_uk^T q_nope) . c_j + q_rot . k_rot_j,
+// out = W_uv (sum_j p_j c_j) — only the latent c_j and the rotated key part are cached, and a portion of a prompt needs nothing
+// of the tokens before it but their cache rows.
+#include <math.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <algorithm>
+#include <map>
+#include <string>
+#include <vector>
+
+#include "lm_kernels.h"
+#include "zg_kernels.h"
+
+namespace zg {
+namespace lm {
+
+namespace {
+
+enum { INIT_MATRIX = 0, INIT_OFFSET = 1, INIT_UNIT = 2, INIT_PLAIN = 3 };
+
+struct Tensor {
+    void* dev = nullptr;
+    bool matrix = false;  // bf16 storage
+    size_t rows = 0, cols = 0;
+    int transpose_heads = 0;  // > 0: source [heads * d][cols] is stored as [heads][cols][d]
+    int init = INIT_MATRIX;
+    bool loaded = false;
+};
+
+struct LayerW {
+    zg_lm_layer d;
+    float *norm1 = nullptr, *norm1b = nullptr, *norm2 = nullptr, *norm2b = nullptr, *shift = nullptr;
+    bf16_t *qfv = nullptr, *o = nullptr;
+    float *fb = nullptr, *lower = nullptr, *hnorm = nullptr;
+    bf16_t *dqkv = nullptr, *uq = nullptr, *ukT = nullptr, *uv = nullptr;
+    float *dq_norm = nullptr, *dkv_norm = nullptr, *rot_freq = nullptr;
+    float rot_amp = 1.0f;
+    bf16_t *up = nullptr, *down = nullptr, *gu = nullptr, *edown = nullptr, *router = nullptr;
+    float* correction = nullptr;
+};
+
+struct Pass {
+    int layer = 0;
+    size_t hgrn_off = 0;     // floats into a slot's recurrent-state block
+    float* cache = nullptr;  // latent cache of this pass
+};
+
+struct Slot {
+    bool open = false;
+    size_t len = 0;
+    std::vector<int> pages;
+};
+
+struct Bump {
+    char* base;
+    size_t off = 0;
+    template <typename T>
+    T* take(size_t n) {
+        off = (off + 255) & ~(size_t)255;
+        T* p = base ? reinterpret_cast<T*>(base + off) : nullptr;
+        off += n * sizeof(T);
+        return p;
+    }
+};
+
+struct Piece {  // the rows one entry contributes to one portion
+    int slot;
+    const int32_t* tok;
+    int n;
+    int pos0;
+    std::vector<std::pair<int, size_t>> wants;  // (row inside the piece, output row)
+};
+
+struct Sampler {
+    float temp;
+    uint64_t seed;
+    int32_t* tokens_out;  // host, indexed by output row
+};
+
+__global__ __launch_bounds__(256) void fill_kernel(void* dst, size_t n, uint64_t key, int kind, float std_) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    uint64_t z = key + (i + 1) * 0x9E3779B97F4A7C15ULL;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ULL;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBULL;
+    z ^= z >> 31;
+    const float s4 = (float)((int)((z & 0xFFFF) + ((z >> 16) & 0xFFFF) + ((z >> 32) & 0xFFFF) + (z >> 48)) - 131070) * (1.0f / 37837.227f);
+    const float u = (float)(uint32_t)(z >> 40) * 5.9604644775390625e-08f;
+    if (kind == INIT_MATRIX) reinterpret_cast<bf16_t*>(dst)[i] = f32_to_bf16_rne(s4 * std_);
+    else if (kind == INIT_OFFSET) reinterpret_cast<float*>(dst)[i] = s4 * 0.05f;
+    else if (kind == INIT_UNIT) reinterpret_cast<float*>(dst)[i] = u;
+    else reinterpret_cast<float*>(dst)[i] = 1.0f + s4 * 0.05f;
+}
+
+__global__ __launch_bounds__(256) void zero_kernel(float* p, size_t n) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0.0f;
+}
+
+}  // namespace
+}  // namespace lm
+}  // namespace zg
+
+using namespace zg;
+using namespace zg::lm;
+
+struct zg_lm {
+    zg_lm_config cfg;
+    std::vector<LayerW> layers;
+    std::vector<Pass> passes;
+    std::map<std::string, Tensor> tensors;
+    int device = 0;
+    hipStream_t stream = nullptr;
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    char* arena = nullptr;
+    size_t arena_bytes = 0;
+    bool f32 = false;
+    int W = 0, V = 0, MS = 0, NS = 0, P = 0, max_pages = 0, n_pages = 0, logit_rows = 0, n_passes = 0;
+    // weights outside the layers
+    bf16_t *embed = nullptr, *head = nullptr;
+    float* final_norm = nullptr;
+    // state
+    float* shift_state = nullptr;  // [NS][passes][W]
+    float* hgrn_state = nullptr;   // [NS][hgrn_floats]
+    size_t hgrn_floats = 0;
+    int* page_table = nullptr;  // [NS][max_pages]
+    std::vector<Slot> slots;
+    std::vector<int> free_pages;
+    // scratch
+    float *x = nullptr, *h = nullptr, *y = nullptr, *proj = nullptr, *cq = nullptr, *q = nullptr, *qa = nullptr, *ctx = nullptr, *o = nullptr, *u = nullptr;
+    float *gu_buf = nullptr, *hb = nullptr, *ye = nullptr, *wt = nullptr, *last_h = nullptr, *hn = nullptr, *logits = nullptr;
+    float *row_max = nullptr, *samp_ws = nullptr, *samp_u = nullptr;
+    int *pick = nullptr, *grp_off = nullptr, *sorted = nullptr, *inv = nullptr, *tok_out = nullptr, *flag = nullptr;
+    int* meta = nullptr;    // device: ids | pos | slot | prev | last-entry | want rows | entry start | entry len | entry slot
+    int* h_meta = nullptr;  // pinned twin
+    float* h_logits = nullptr;  // pinned [logit_rows][V]
+    int* h_small = nullptr;     // pinned: sampled tokens [logit_rows], fault flag
+    float* h_u = nullptr;       // pinned uniforms [logit_rows]
+    float* trace = nullptr;
+    size_t trace_floats = 0;
+    float last_step_ms = 0.0f, last_decode_ms = 0.0f;
+};
+
+namespace {
+
+size_t meta_ints(const zg_lm* g) { return (size_t)6 * g->MS + (size_t)3 * g->NS; }
+
+// Everything that lives in the arena, in one place: called once with a null base to measure and once to place.
+void layout(zg_lm* g, Bump& b) {
+    const size_t W = g->W, V = g->V, MS = g->MS, NS = g->NS;
+    auto& T = g->tensors;
+    T.clear();
+    auto mat = [&](const std::string& name, bf16_t* base, size_t row0, size_t rows, size_t cols, int transpose_heads = 0) {
+        Tensor t;
+        t.dev = base ? base + row0 * cols : nullptr;
+        t.matrix = true;
+        t.rows = rows;
+        t.cols = cols;
+        t.transpose_heads = transpose_heads;
+        t.init = INIT_MATRIX;
+        T[name] = t;
+    };
+    auto vec = [&](const std::string& name, float*& p, size_t n, int init) {
+        p = b.take<float>(n);
+        Tensor t;
+        t.dev = p;
+        t.rows = 1;
+        t.cols = n;
+        t.init = init;
+        T[name] = t;
+    };
+    g->embed = b.take<bf16_t>(V * W);
+    mat("embed", g->embed, 0, V, W);
+    g->head = b.take<bf16_t>(V * W);
+    mat("head", g->head, 0, V, W);
+    vec("final.norm", g->final_norm, W, INIT_OFFSET);
+    size_t max_proj = 1, max_qr = 1, max_q = 1, max_qa = 1, max_ctx = 1, max_o = 1, max_ff = 1, max_assign = 1, max_gu = 1, max_hb = 1, max_e = 1;
+    for (size_t i = 0; i < g->layers.size(); ++i) {
+        LayerW& L = g->layers[i];
+        const zg_lm_layer& d = L.d;
+        const std::string p = "l" + std::to_string(i) + ".";
+        vec(p + "norm1", L.norm1, W, INIT_OFFSET);
+        vec(p + "norm1b", L.norm1b, W, INIT_OFFSET);
+        vec(p + "shift", L.shift, W, INIT_UNIT);
+        const size_t H = d.heads, D = d.dim, Vd = d.vdim;
+        if (d.mixer == ZG_LM_MIX_HGRN2) {
+            const size_t HD = H * D, HV = H * Vd;
+            L.qfv = b.take<bf16_t>((2 * HD + HV) * W);
+            mat(p + "mix.q", L.qfv, 0, HD, W);
+            mat(p + "mix.f", L.qfv, HD, HD, W);
+            mat(p + "mix.v", L.qfv, 2 * HD, HV, W);
+            vec(p + "mix.f.b", L.fb, HD, INIT_OFFSET);
+            vec(p + "mix.lower", L.lower, HD, INIT_UNIT);
+            vec(p + "mix.norm", L.hnorm, Vd, INIT_PLAIN);
+            L.o = b.take<bf16_t>(W * HV);
+            mat(p + "mix.o", L.o, 0, W, HV);
+            max_proj = std::max(max_proj, 2 * HD + HV);
+            max_o = std::max(max_o, HV);
+        } else {
+            const size_t R = d.rot_dim, KR = d.kv_rank, QR = d.q_rank, HV = H * Vd;
+            L.dqkv = b.take<bf16_t>((QR + KR + R) * W);
+            mat(p + "mix.dq", L.dqkv, 0, QR, W);
+            mat(p + "mix.dkv", L.dqkv, QR, KR + R, W);
+            vec(p + "mix.dq.norm", L.dq_norm, QR, INIT_PLAIN);
+            vec(p + "mix.dkv.norm", L.dkv_norm, KR, INIT_PLAIN);
+            L.uq = b.take<bf16_t>(H * (D + R) * QR);
+            mat(p + "mix.uq", L.uq, 0, H * (D + R), QR);
+            L.ukT = b.take<bf16_t>(H * KR * D);
+            mat(p + "mix.uk", L.ukT, 0, H * D, KR, (int)H);
+            L.uv = b.take<bf16_t>(HV * KR);
+            mat(p + "mix.uv", L.uv, 0, HV, KR);
+            L.o = b.take<bf16_t>(W * HV);
+            mat(p + "mix.o", L.o, 0, W, HV);
+            L.rot_freq = b.take<float>(std::max<size_t>(1, d.rot_dims / 2));
+            max_proj = std::max(max_proj, QR + KR + R);
+            max_qr = std::max(max_qr, QR);
+            max_q = std::max(max_q, H * (D + R));
+            max_qa = std::max(max_qa, H * (KR + R));
+            max_ctx = std::max(max_ctx, H * KR);
+            max_o = std::max(max_o, HV);
+        }
+        if (d.ff != ZG_LM_FF_NONE) {
+            vec(p + "norm2", L.norm2, W, INIT_OFFSET);
+            vec(p + "norm2b", L.norm2b, W, INIT_OFFSET);
+        }
+        const size_t F = d.ff_width;
+        if (d.ff == ZG_LM_FF_DENSE) {
+            L.up = b.take<bf16_t>(F * W);
+            mat(p + "mlp.up", L.up, 0, F, W);
+            L.down = b.take<bf16_t>(W * F);
+            mat(p + "mlp.down", L.down, 0, W, F);
+            max_ff = std::max(max_ff, F);
+        } else if (d.ff == ZG_LM_FF_MOE) {
+            const size_t E = d.experts;
+            L.gu = b.take<bf16_t>(E * 2 * F * W);
+            L.edown = b.take<bf16_t>(E * W * F);
+            for (size_t e = 0; e < E; ++e) {
+                const std::string q = p + "mlp.e" + std::to_string(e) + ".";
+                mat(q + "gate", L.gu, e * 2 * F, F, W);
+                mat(q + "up", L.gu, e * 2 * F + F, F, W);
+                mat(q + "down", L.edown, e * W, W, F);
+            }
+            L.router = b.take<bf16_t>(E * W);
+            mat(p + "mlp.router", L.router, 0, E, W);
+            vec(p + "mlp.correction", L.correction, E, INIT_OFFSET);
+            max_assign = std::max(max_assign, (size_t)d.top);
+            max_gu = std::max(max_gu, (size_t)d.top * 2 * F);
+            max_hb = std::max(max_hb, (size_t)d.top * F);
+            max_e = std::max(max_e, E);
+        }
+    }
+    // state
+    g->shift_state = b.take<float>(NS * g->n_passes * W);
+    size_t hg = 0;
+    for (Pass& ps : g->passes) {
+        const zg_lm_layer& d = g->layers[ps.layer].d;
+        if (d.mixer == ZG_LM_MIX_HGRN2) {
+            ps.hgrn_off = hg;
+            hg += (size_t)d.heads * d.dim * d.vdim;
+        }
+    }
+    g->hgrn_floats = hg;
+    g->hgrn_state = b.take<float>(std::max<size_t>(1, NS * hg));
+    g->page_table = b.take<int>(NS * g->max_pages);
+    for (Pass& ps : g->passes) {
+        const zg_lm_layer& d = g->layers[ps.layer].d;
+        if (d.mixer == ZG_LM_MIX_LATENT_ATTENTION) ps.cache = b.take<float>((size_t)g->n_pages * g->P * (d.kv_rank + d.rot_dim));
+    }
+    // scratch
+    g->x = b.take<float>(MS * W);
+    g->h = b.take<float>(MS * W);
+    g->y = b.take<float>(MS * W);
+    g->proj = b.take<float>(MS * max_proj);
+    g->cq = b.take<float>(MS * max_qr);
+    g->q = b.take<float>(MS * max_q);
+    g->qa = b.take<float>(MS * max_qa);
+    g->ctx = b.take<float>(MS * max_ctx);
+    g->o = b.take<float>(MS * max_o);
+    g->u = b.take<float>(MS * max_ff);
+    g->gu_buf = b.take<float>(MS * max_gu);
+    g->hb = b.take<float>(MS * max_hb);
+    g->ye = b.take<float>(MS * max_assign * W);
+    g->wt = b.take<float>(MS * max_assign);
+    g->pick = b.take<int>(MS * max_assign);
+    g->sorted = b.take<int>(MS * max_assign);
+    g->inv = b.take<int>(MS * max_assign);
+    g->grp_off = b.take<int>(max_e + 1);
+    g->last_h = b.take<float>((size_t)g->n_passes * NS * W);
+    g->hn = b.take<float>((size_t)g->logit_rows * W);
+    g->logits = b.take<float>((size_t)g->logit_rows * V);
+    g->row_max = b.take<float>(g->logit_rows);
+    g->samp_ws = b.take<float>(sample_workspace_floats(g->logit_rows));
+    g->samp_u = b.take<float>(g->logit_rows);
+    g->tok_out = b.take<int>(g->logit_rows);
+    g->flag = b.take<int>(16);
+    g->meta = b.take<int>(meta_ints(g));
+}
+
+// YaRN blend of the rotary frequencies (host, double): pairs below `lo` keep their frequency, pairs above `hi` are slowed by
+// `factor`, a linear ramp between; the amplitude factor multiplies cos and sin.
+void rotary_table(const zg_lm_layer& d, std::vector<float>& freq, float& amp) {
+    const int dims = d.rot_dims, half = dims / 2;
+    freq.resize(std::max(1, half));
+    amp = 1.0f;
+    double lo = 0, hi = 0;
+    if (d.rot_scaled) {
+        auto corr = [&](double t) { return dims * log((double)d.rot_original / (2.0 * M_PI * t)) / (2.0 * log((double)d.rot_base)); };
+        lo = std::max(floor(corr(d.rot_fast)), 0.0);
+        hi = std::min(ceil(corr(d.rot_slow)), (double)dims - 1.0);
+        amp = (float)(0.1 * log((double)d.rot_factor) + 1.0);
+    }
+    for (int i = 0; i < half; ++i) {
+        double f = pow((double)d.rot_base, -2.0 * i / dims);
+        if (d.rot_scaled) {
+            const double ramp = std::min(1.0, std::max(0.0, (i - lo) / std::max(hi - lo, 0.001)));
+            f = f / d.rot_factor * ramp + f * (1.0 - ramp);
+        }
+        freq[i] = (float)f;
+    }
+}
+
+int check_layer(const zg_lm_layer& d, size_t i) {
+    ZG_REQUIRE(d.mixer == ZG_LM_MIX_HGRN2 || d.mixer == ZG_LM_MIX_LATENT_ATTENTION, ZG_ERR_ARG, "layer %zu: unknown mixer %d", i, d.mixer);
+    ZG_REQUIRE(d.heads >= 1 && d.dim >= 1 && d.vdim >= 1, ZG_ERR_ARG, "layer %zu: heads %d dim %d vdim %d", i, d.heads, d.dim, d.vdim);
+    if (d.mixer == ZG_LM_MIX_HGRN2) {
+        ZG_REQUIRE(d.dim <= 256, ZG_ERR_UNSUPPORTED, "layer %zu: %d key channels per head of the recurrence (at most 256)", i, d.dim);
+    } else {
+        ZG_REQUIRE(d.rot_dim >= 0 && d.kv_rank >= 1 && d.q_rank >= 1, ZG_ERR_ARG, "layer %zu: rot_dim %d kv_rank %d q_rank %d", i, d.rot_dim,
+                   d.kv_rank, d.q_rank);
+        ZG_REQUIRE(d.rot_dims >= 0 && d.rot_dims % 2 == 0 && d.rot_dims <= d.rot_dim, ZG_ERR_ARG, "layer %zu: %d rotated dimensions of %d", i,
+                   d.rot_dims, d.rot_dim);
+        ZG_REQUIRE(d.kv_rank + d.rot_dim <= 1024, ZG_ERR_UNSUPPORTED, "layer %zu: %d cached dimensions per token (at most 1024)", i,
+                   d.kv_rank + d.rot_dim);
+        ZG_REQUIRE(d.rot_dims == 0 || d.rot_base > 0.0f, ZG_ERR_ARG, "layer %zu: rotary base %f", i, d.rot_base);
+        ZG_REQUIRE(!d.rot_scaled || (d.rot_factor > 0.0f && d.rot_original > 0.0f && d.rot_fast > 0.0f && d.rot_slow > 0.0f), ZG_ERR_ARG,
+                   "layer %zu: rotary scaling constants must be positive", i);
+    }
+    ZG_REQUIRE(d.ff == ZG_LM_FF_NONE || d.ff == ZG_LM_FF_DENSE || d.ff == ZG_LM_FF_MOE, ZG_ERR_ARG, "layer %zu: unknown feed-forward %d", i, d.ff);
+    ZG_REQUIRE(d.ff == ZG_LM_FF_NONE || d.ff_width >= 1, ZG_ERR_ARG, "layer %zu: feed-forward width %d", i, d.ff_width);
+    ZG_REQUIRE(d.ff != ZG_LM_FF_MOE || (d.experts >= 1 && d.experts <= 256 && d.top >= 1 && d.top <= d.experts), ZG_ERR_UNSUPPORTED,
+               "layer %zu: %d experts, %d chosen (at most 256 experts)", i, d.experts, d.top);
+    return ZG_OK;
+}
+
+// ------------------------------------------------------------------------------------------------ one portion of rows
+int run_portion(zg_lm* g, const std::vector<Piece>& pieces, float* logits_out, const Sampler* sampler) {
+    hipStream_t s = g->stream;
+    const int W = g->W, MS = g->MS, NS = g->NS;
+    int M = 0;
+    for (const Piece& pc : pieces) M += pc.n;
+    if (M == 0) return ZG_OK;
+    const int n_ent = (int)pieces.size();
+    int *ids = g->h_meta, *pos = ids + MS, *slot = pos + MS, *prev = slot + MS, *lastent = prev + MS, *want_rows = lastent + MS;
+    int *ent_start = want_rows + MS, *ent_len = ent_start + NS, *ent_slot = ent_len + NS;
+    std::vector<std::pair<int, size_t>> wants;  // (row of the portion, output row)
+    int r = 0;
+    for (int e = 0; e < n_ent; ++e) {
+        const Piece& pc = pieces[e];
+        ent_start[e] = r;
+        ent_len[e] = pc.n;
+        ent_slot[e] = pc.slot;
+        for (int t = 0; t < pc.n; ++t, ++r) {
+            ids[r] = pc.tok[t];
+            pos[r] = pc.pos0 + t;
+            slot[r] = pc.slot;
+            prev[r] = t > 0 ? r - 1 : -1;
+            lastent[r] = t == pc.n - 1 ? e : -1;
+        }
+        for (auto& w : pc.wants) wants.push_back({ent_start[e] + w.first, w.second});
+        const Slot& sl = g->slots[pc.slot];
+        ZG_HIP(hipMemcpyAsync(g->page_table + (size_t)pc.slot * g->max_pages, sl.pages.data(), sl.pages.size() * sizeof(int), hipMemcpyHostToDevice, s));
+    }
+    ZG_HIP(hipMemcpyAsync(g->meta, g->h_meta, meta_ints(g) * sizeof(int), hipMemcpyHostToDevice, s));
+    const int *d_ids = g->meta, *d_pos = d_ids + MS, *d_slot = d_pos + MS, *d_prev = d_slot + MS, *d_last = d_prev + MS, *d_want = d_last + MS;
+    const int *d_estart = d_want + MS, *d_elen = d_estart + NS, *d_eslot = d_elen + NS;
+    const bool f32 = g->f32;
+    const float eps = g->cfg.norm_eps;
+    const bool few = M <= kGemvMaxRows;
+
+    ZG_HIP(hipEventRecord(g->ev0, s));
+    ZG_TRY(launch_embed(g->embed, d_ids, g->x, M, W, g->V, g->flag, s));
+    for (int p = 0; p < g->n_passes; ++p) {
+        const Pass& ps = g->passes[p];
+        const LayerW& L = g->layers[ps.layer];
+        const zg_lm_layer& d = L.d;
+        const int H = d.heads, D = d.dim, Vd = d.vdim;
+        ZG_TRY(launch_norm_shift(g->x, L.norm1, L.shift, eps, g->h, M, W, d_prev, d_slot, g->shift_state + (size_t)p * W, (size_t)g->n_passes * W,
+                                 d_last, g->last_h + (size_t)p * NS * W, s));
+        Linear lin;
+        if (d.mixer == ZG_LM_MIX_HGRN2) {
+            const int HD = H * D, HV = H * Vd, NP = 2 * HD + HV;
+            lin = Linear();
+            lin.A = g->h; lin.lda = W; lin.B = L.qfv; lin.ldb = W; lin.C = g->proj; lin.ldc = NP; lin.M = M; lin.N = NP; lin.K = W;
+            ZG_TRY(launch_linear(lin, f32, s));
+            ZG_TRY(launch_hgrn2_gates(g->proj, NP, M, HD, L.fb, L.lower, s));
+            ZG_TRY(launch_hgrn2_scan(g->proj, NP, g->o, HV, g->hgrn_state + ps.hgrn_off, g->hgrn_floats, d_estart, d_elen, d_eslot, n_ent, H, D, Vd, s));
+            ZG_TRY(launch_norm_plain(g->o, HV, H, Vd, M, L.hnorm, eps, s));
+            lin = Linear();
+            lin.A = g->o; lin.lda = HV; lin.B = L.o; lin.ldb = HV; lin.C = g->y; lin.ldc = W; lin.M = M; lin.N = W; lin.K = HV;
+            ZG_TRY(launch_linear(lin, f32, s));
+        } else {
+            const int R = d.rot_dim, KR = d.kv_rank, QR = d.q_rank, HV = H * Vd, NP = QR + KR + R;
+            const Rotary rot{L.rot_freq, d.rot_dims, L.rot_amp};
+            lin = Linear();
+            lin.A = g->h; lin.lda = W; lin.B = L.dqkv; lin.ldb = W; lin.C = g->proj; lin.ldc = NP; lin.M = M; lin.N = NP; lin.K = W;
+            ZG_TRY(launch_linear(lin, f32, s));
+            ZG_TRY(launch_latent_prep(g->proj, NP, M, QR, KR, R, L.dq_norm, L.dkv_norm, eps, rot, d_pos, d_slot, g->page_table, g->max_pages, g->P,
+                                      g->cq, ps.cache, s));
+            lin = Linear();
+            lin.A = g->cq; lin.lda = QR; lin.B = L.uq; lin.ldb = QR; lin.C = g->q; lin.ldc = H * (D + R); lin.M = M; lin.N = H * (D + R); lin.K = QR;
+            ZG_TRY(launch_linear(lin, f32, s));
+            lin = Linear();  // the unrotated query part carried into the latent space, head by head
+            lin.A = g->q; lin.lda = H * (D + R); lin.a_zoff = D + R; lin.B = L.ukT; lin.ldb = D; lin.b_zoff = (long long)KR * D;
+            lin.C = g->qa; lin.ldc = H * (KR + R); lin.c_zoff = KR + R; lin.M = M; lin.N = KR; lin.K = D; lin.nz = H;
+            ZG_TRY(launch_linear(lin, f32, s));
+            ZG_TRY(launch_q_rotary(g->q, H * (D + R), g->qa, H * (KR + R), M, H, D, R, KR, rot, d_pos, s));
+            ZG_TRY(launch_latent_attention(g->qa, g->ctx, M, H, KR, R, d.scale, d_pos, d_slot, g->page_table, g->max_pages, g->P, ps.cache, nullptr, 0, s));
+            lin = Linear();  // values of the weighted latent, head by head
+            lin.A = g->ctx; lin.lda = H * KR; lin.a_zoff = KR; lin.B = L.uv; lin.ldb = KR; lin.b_zoff = (long long)Vd * KR;
+            lin.C = g->o; lin.ldc = HV; lin.c_zoff = Vd; lin.M = M; lin.N = Vd; lin.K = KR; lin.nz = H;
+            ZG_TRY(launch_linear(lin, f32, s));
+            lin = Linear();
+            lin.A = g->o; lin.lda = HV; lin.B = L.o; lin.ldb = HV; lin.C = g->y; lin.ldc = W; lin.M = M; lin.N = W; lin.K = HV;
+            ZG_TRY(launch_linear(lin, f32, s));
+        }
+        ZG_TRY(launch_norm_add(g->x, g->y, L.norm1b, eps, M, W, s));
+        if (d.ff != ZG_LM_FF_NONE)
+            ZG_TRY(launch_norm_shift(g->x, L.norm2, nullptr, eps, g->h, M, W, nullptr, nullptr, nullptr, 0, nullptr, nullptr, s));
+        const int F = d.ff_width;
+        if (d.ff == ZG_LM_FF_DENSE) {
+            lin = Linear();
+            lin.A = g->h; lin.lda = W; lin.B = L.up; lin.ldb = W; lin.C = g->u; lin.ldc = F; lin.M = M; lin.N = F; lin.K = W; lin.act = ACT_RELU2;
+            ZG_TRY(launch_linear(lin, f32, s));
+            lin = Linear();
+            lin.A = g->u; lin.lda = F; lin.B = L.down; lin.ldb = F; lin.C = g->y; lin.ldc = W; lin.M = M; lin.N = W; lin.K = F;
+            ZG_TRY(launch_linear(lin, f32, s));
+            ZG_TRY(launch_norm_add(g->x, g->y, L.norm2b, eps, M, W, s));
+        } else if (d.ff == ZG_LM_FF_MOE) {
+            const int E = d.experts, top = d.top, NA = M * top;
+            ZG_TRY(launch_route(g->h, M, W, L.router, L.correction, E, top, g->pick, g->wt, s));
+            Linear up, dn;
+            up.A = g->h; up.lda = W; up.a_div = top; up.B = L.gu; up.ldb = W; up.b_zoff = (long long)2 * F * W; up.C = g->gu_buf; up.ldc = 2 * F;
+            up.N = 2 * F; up.K = W;
+            dn.A = g->hb; dn.lda = F; dn.B = L.edown; dn.ldb = F; dn.b_zoff = (long long)W * F; dn.C = g->ye; dn.ldc = W; dn.N = W; dn.K = F;
+            if (few) {  // one batch per assignment, its expert's matrices looked up on the device
+                up.M = dn.M = 1; up.nz = dn.nz = NA; up.z_group = dn.z_group = g->pick;
+                up.c_zoff = 2 * F; dn.c_zoff = W;
+            } else {  // assignments sorted by expert, grouped products
+                ZG_TRY(launch_group(g->pick, NA, E, g->grp_off, g->sorted, g->inv, s));
+                up.M = dn.M = NA; up.a_rows = g->sorted; up.grp_off = dn.grp_off = g->grp_off; up.n_groups = dn.n_groups = E;
+            }
+            ZG_TRY(launch_linear(up, f32, s));
+            ZG_TRY(launch_glu(g->gu_buf, g->hb, NA, F, s));
+            ZG_TRY(launch_linear(dn, f32, s));
+            ZG_TRY(launch_moe_combine(g->x, g->ye, few ? nullptr : g->inv, g->wt, top, L.norm2b, eps, M, W, s));
+        }
+        if (g->trace && (size_t)(p + 1) * M * W <= g->trace_floats) {
+            ZG_HIP(hipMemcpyAsync(g->trace + (size_t)p * M * W, g->x, (size_t)M * W * sizeof(float), hipMemcpyDeviceToHost, s));
+            ZG_HIP(hipStreamSynchronize(s));
+        }
+    }
+    // the rows the last tokens of the entries left for the token shift of their successors
+    ZG_TRY(launch_commit_rows(g->shift_state, (size_t)g->n_passes * W, g->last_h, W, d_eslot, n_ent, W, g->n_passes, W, (size_t)NS * W, s));
+
+    // logits of the rows that were asked for, logit_rows at a time
+    size_t w0 = 0;
+    do {
+        const int nw = (int)std::min<size_t>(g->logit_rows, wants.size() - w0);
+        if (nw > 0) {
+            // (the want rows travel through the pinned twin of the metadata; the stream is drained at the end of every batch,
+            // so the twin is free again when the next batch fills it)
+            for (int j = 0; j < nw; ++j) want_rows[j] = wants[w0 + j].first;
+            ZG_HIP(hipMemcpyAsync(g->meta + 5 * (size_t)MS, want_rows, nw * sizeof(int), hipMemcpyHostToDevice, s));
+            ZG_TRY(launch_norm_gather(g->x, d_want, g->final_norm, eps, g->hn, nw, W, s));
+            Linear lin;
+            lin.A = g->hn; lin.lda = W; lin.B = g->head; lin.ldb = W; lin.C = g->logits; lin.ldc = g->V; lin.M = nw; lin.N = g->V; lin.K = W;
+            ZG_TRY(launch_linear(lin, f32, s));
+            if (sampler) {
+                ZG_TRY(launch_row_argmax(g->logits, nw, g->V, g->row_max, g->tok_out, s));
+                if (sampler->temp > 0.0f) {
+                    for (int j = 0; j < nw; ++j) {  // the uniform of (seed, length of the sequence with the token to be drawn, output row)
+                        const int row = wants[w0 + j].first;
+                        uint64_t z = sampler->seed * 0x9E3779B97F4A7C15ULL + (uint64_t)(pos[row] + 2) * 0xD1B54A32D192ED03ULL + wants[w0 + j].second + 1;
+                        z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ULL;
+                        z = (z ^ (z >> 27)) * 0x94D049BB133111EBULL;
+                        z ^= z >> 31;
+                        g->h_u[j] = (float)(uint32_t)(z >> 40) * 5.9604644775390625e-08f;
+                    }
+                    ZG_HIP(hipMemcpyAsync(g->samp_u, g->h_u, nw * sizeof(float), hipMemcpyHostToDevice, s));
+                    ZG_TRY(launch_sample(g->logits, nw, g->V, sampler->temp, g->samp_u, g->row_max, 1, 1, g->samp_ws, g->tok_out, false, s));
+                }
+                ZG_HIP(hipMemcpyAsync(g->h_small, g->tok_out, nw * sizeof(int), hipMemcpyDeviceToHost, s));
+            } else if (logits_out) {
+                ZG_HIP(hipMemcpyAsync(g->h_logits, g->logits, (size_t)nw * g->V * sizeof(float), hipMemcpyDeviceToHost, s));
+            }
+        }
+        if (w0 + nw >= wants.size()) ZG_HIP(hipEventRecord(g->ev1, s));
+        ZG_HIP(hipMemcpyAsync(g->h_small + g->logit_rows, g->flag, sizeof(int), hipMemcpyDeviceToHost, s));
+        ZG_HIP(hipStreamSynchronize(s));
+        for (int j = 0; j < nw; ++j) {
+            const size_t out_row = wants[w0 + j].second;
+            if (sampler) sampler->tokens_out[out_row] = g->h_small[j];
+            else if (logits_out) memcpy(logits_out + out_row * g->V, g->h_logits + (size_t)j * g->V, (size_t)g->V * sizeof(float));
+        }
+        w0 += nw;
+    } while (w0 < wants.size());
+    float ms = 0.0f;
+    ZG_HIP(hipEventElapsedTime(&ms, g->ev0, g->ev1));
+    g->last_step_ms += ms;
+    ZG_REQUIRE(g->h_small[g->logit_rows] == 0, ZG_ERR_ARG, "step: a token id outside the vocabulary of %d", g->V);
+    return ZG_OK;
+}
+
+int step_impl(zg_lm* g, const zg_lm_entry* entries, size_t n_entries, float* logits_out, size_t logits_len, const Sampler* sampler) {
+    ZG_REQUIRE(g && (entries || n_entries == 0), ZG_ERR_ARG, "lm_step: bad argument");
+    ZG_HIP(hipSetDevice(g->device));
+    size_t n_want = 0, need_pages = 0;
+    for (size_t i = 0; i < n_entries; ++i) {
+        const zg_lm_entry& e = entries[i];
+        ZG_REQUIRE(e.seq >= 0 && e.seq < g->NS && g->slots[e.seq].open, ZG_ERR_ARG, "lm_step: entry %zu names sequence %d, which is not open", i, e.seq);
+        for (size_t j = 0; j < i; ++j) ZG_REQUIRE(entries[j].seq != e.seq, ZG_ERR_ARG, "lm_step: sequence %d appears in two entries", e.seq);
+        ZG_REQUIRE(e.n_tokens == 0 || e.tokens, ZG_ERR_ARG, "lm_step: entry %zu has no tokens", i);
+        ZG_REQUIRE(e.n_want == 0 || e.want, ZG_ERR_ARG, "lm_step: entry %zu has no want list", i);
+        for (size_t t = 0; t < e.n_tokens; ++t)
+            ZG_REQUIRE(e.tokens[t] >= 0 && e.tokens[t] < g->V, ZG_ERR_ARG, "lm_step: token %d outside the vocabulary of %d", e.tokens[t], g->V);
+        for (size_t j = 0; j < e.n_want; ++j)
+            ZG_REQUIRE(e.want[j] >= 0 && (size_t)e.want[j] < e.n_tokens, ZG_ERR_ARG, "lm_step: entry %zu asks for place %d of %zu tokens", i, e.want[j],
+                       e.n_tokens);
+        n_want += e.n_want;
+        const Slot& sl = g->slots[e.seq];
+        const size_t pages = (sl.len + e.n_tokens + g->P - 1) / g->P;
+        ZG_REQUIRE(pages <= (size_t)g->max_pages, ZG_ERR_SHAPE, "lm_step: sequence %d would hold %zu tokens (at most %zu)", e.seq, sl.len + e.n_tokens,
+                   (size_t)g->max_pages * g->P);
+        need_pages += pages > sl.pages.size() ? pages - sl.pages.size() : 0;
+    }
+    ZG_REQUIRE(need_pages <= g->free_pages.size(), ZG_ERR_SHAPE, "lm_step: %zu cache pages needed, %zu free (max_tokens %zu)", need_pages,
+               g->free_pages.size(), g->cfg.max_tokens);
+    ZG_REQUIRE(sampler || n_want == 0 || (logits_out && logits_len >= n_want * (size_t)g->V), ZG_ERR_SHAPE, "lm_step: logits_out needs %zu elements",
+               n_want * (size_t)g->V);
+    for (size_t i = 0; i < n_entries; ++i) {
+        Slot& sl = g->slots[entries[i].seq];
+        const size_t pages = (sl.len + entries[i].n_tokens + g->P - 1) / g->P;
+        while (sl.pages.size() < pages) {
+            sl.pages.push_back(g->free_pages.back());
+            g->free_pages.pop_back();
+        }
+    }
+    g->last_step_ms = 0.0f;
+    // cut the entries into portions of at most max_step_tokens rows
+    std::vector<Piece> pieces;
+    int rows = 0;
+    size_t out_base = 0;
+    for (size_t i = 0; i < n_entries; ++i) {
+        const zg_lm_entry& e = entries[i];
+        Slot& sl = g->slots[e.seq];
+        size_t done = 0;
+        while (done < e.n_tokens) {
+            const int n = (int)std::min<size_t>(e.n_tokens - done, (size_t)(g->MS - rows));
+            Piece pc;
+            pc.slot = e.seq;
+            pc.tok = e.tokens + done;
+            pc.n = n;
+            pc.pos0 = (int)(sl.len + done);
+            for (size_t j = 0; j < e.n_want; ++j)
+                if ((size_t)e.want[j] >= done && (size_t)e.want[j] < done + n) pc.wants.push_back({(int)(e.want[j] - done), out_base + j});
+            pieces.push_back(pc);
+            rows += n;
+            done += n;
+            if (rows == g->MS) {
+                ZG_TRY(run_portion(g, pieces, logits_out, sampler));
+                pieces.clear();
+                rows = 0;
+            }
+        }
+        sl.len += e.n_tokens;
+        out_base += e.n_want;
+    }
+    if (!pieces.empty()) ZG_TRY(run_portion(g, pieces, logits_out, sampler));
+    return ZG_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int zg_lm_create(zg_lm** out, const zg_lm_config* config, int device) {
+    ZG_REQUIRE(out && config && config->layers && config->n_layers >= 1, ZG_ERR_ARG, "lm_create: bad argument");
+    ZG_REQUIRE(config->vocab >= 1 && config->width >= 1 && config->vocab <= 262144, ZG_ERR_ARG, "lm_create: vocab %zu width %zu", config->vocab,
+               config->width);
+    ZG_REQUIRE(config->norm_eps >= 0.0f, ZG_ERR_ARG, "lm_create: norm eps %g", config->norm_eps);
+    int n_dev = 0;
+    ZG_HIP(hipGetDeviceCount(&n_dev));
+    ZG_REQUIRE(device >= 0 && device < n_dev, ZG_ERR_ARG, "device %d out of range (%d visible)", device, n_dev);
+    ZG_HIP(hipSetDevice(device));
+    hipDeviceProp_t prop;
+    ZG_HIP(hipGetDeviceProperties(&prop, device));
+    ZG_REQUIRE(strncmp(prop.gcnArchName, "gfx950", 6) == 0, ZG_ERR_UNSUPPORTED, "built for gfx950 (MI355X) only; device %d is %s", device,
+               prop.gcnArchName);
+    zg_lm* g = new zg_lm();
+    g->cfg = *config;
+    g->device = device;
+    g->f32 = (config->flags & ZG_LM_F32) != 0;
+    g->W = (int)config->width;
+    g->V = (int)config->vocab;
+    g->MS = (int)(config->max_step_tokens ? config->max_step_tokens : 2048);
+    g->NS = (int)std::max<size_t>(1, config->max_seqs);
+    g->P = (int)(config->page_tokens ? config->page_tokens : 64);
+    const size_t max_tokens = std::max<size_t>(1, config->max_tokens);
+    g->max_pages = (int)((max_tokens + g->P - 1) / g->P);
+    g->n_pages = g->max_pages + g->NS;  // every open sequence may leave one page partly used
+    g->logit_rows = std::min(g->MS, 256);
+    int status = ZG_OK;
+    for (size_t i = 0; i < config->n_layers && status == ZG_OK; ++i) {
+        status = check_layer(config->layers[i], i);
+        LayerW L;
+        L.d = config->layers[i];
+        g->layers.push_back(L);
+    }
+    g->cfg.layers = nullptr;
+    const int n = (int)config->n_layers;
+    int a = 0, b = 0, k = 1;
+    if (status == ZG_OK && config->loop_times > 1) {
+        a = config->loop_start; b = config->loop_stop; k = config->loop_times;
+        if (!(a >= 0 && a <= b && b <= n)) {
+            set_error("lm_create: loop [%d, %d) outside the %d layers", a, b, n);
+            status = ZG_ERR_ARG;
+        }
+    }
+    if (status != ZG_OK) {
+        delete g;
+        return status;
+    }
+    auto add = [&](int layer) {
+        Pass ps;
+        ps.layer = layer;
+        g->passes.push_back(ps);
+    };
+    for (int i = 0; i < a; ++i) add(i);
+    for (int t = 0; t < k; ++t)
+        for (int i = a; i < b; ++i) add(i);
+    for (int i = (k > 1 ? b : 0); i < n; ++i) add(i);
+    g->n_passes = (int)g->passes.size();
+    Bump measure{nullptr};
+    layout(g, measure);
+    g->arena_bytes = measure.off + 256;
+    auto fail = [&](int code) {
+        zg_lm_destroy(g);
+        return code;
+    };
+    if (hipMalloc(reinterpret_cast<void**>(&g->arena), g->arena_bytes) != hipSuccess) {
+        (void)hipGetLastError();
+        set_error("lm_create: %zu bytes of device memory not available", g->arena_bytes);
+        g->arena = nullptr;
+        return fail(ZG_ERR_HIP);
+    }
+    Bump place{g->arena};
+    layout(g, place);
+#define ZG_LM_TRY_HIP(expr)                                       \
+    do {                                                          \
+        hipError_t _e = (expr);                                   \
+        if (_e != hipSuccess) return fail(hip_fail(_e, #expr, __FILE__, __LINE__)); \
+    } while (0)
+    ZG_LM_TRY_HIP(hipStreamCreateWithFlags(&g->stream, hipStreamNonBlocking));
+    ZG_LM_TRY_HIP(hipEventCreate(&g->ev0));
+    ZG_LM_TRY_HIP(hipEventCreate(&g->ev1));
+    ZG_LM_TRY_HIP(hipHostMalloc(reinterpret_cast<void**>(&g->h_meta), meta_ints(g) * sizeof(int), hipHostMallocDefault));
+    ZG_LM_TRY_HIP(hipHostMalloc(reinterpret_cast<void**>(&g->h_logits), (size_t)g->logit_rows * g->V * sizeof(float), hipHostMallocDefault));
+    ZG_LM_TRY_HIP(hipHostMalloc(reinterpret_cast<void**>(&g->h_small), (g->logit_rows + 16) * sizeof(int), hipHostMallocDefault));
+    ZG_LM_TRY_HIP(hipHostMalloc(reinterpret_cast<void**>(&g->h_u), g->logit_rows * sizeof(float), hipHostMallocDefault));
+    memset(g->h_meta, 0, meta_ints(g) * sizeof(int));
+    // state and flags start at zero; rotary tables
+    const size_t state_floats = (size_t)g->NS * g->n_passes * g->W;
+    zero_kernel<<<(unsigned)((state_floats + 255) / 256), 256, 0, g->stream>>>(g->shift_state, state_floats);
+    zero_kernel<<<1, 256, 0, g->stream>>>(reinterpret_cast<float*>(g->flag), 16);
+    zero_kernel<<<(unsigned)(((size_t)g->NS * g->max_pages + 255) / 256), 256, 0, g->stream>>>(reinterpret_cast<float*>(g->page_table),
+                                                                                            (size_t)g->NS * g->max_pages);
+    for (LayerW& L : g->layers)
+        if (L.d.mixer == ZG_LM_MIX_LATENT_ATTENTION) {
+            std::vector<float> freq;
+            rotary_table(L.d, freq, L.rot_amp);
+            ZG_LM_TRY_HIP(hipMemcpy(L.rot_freq, freq.data(), std::max<size_t>(1, L.d.rot_dims / 2) * sizeof(float), hipMemcpyHostToDevice));
+        }
+    ZG_LM_TRY_HIP(hipStreamSynchronize(g->stream));
+#undef ZG_LM_TRY_HIP
+    g->slots.assign(g->NS, Slot());
+    for (int p = g->n_pages - 1; p >= 0; --p) g->free_pages.push_back(p);
+    *out = g;
+    return ZG_OK;
+}
+
+int zg_lm_destroy(zg_lm* g) {
+    if (!g) return ZG_OK;
+    (void)hipSetDevice(g->device);
+    if (g->stream) (void)hipStreamSynchronize(g->stream);
+    if (g->ev0) (void)hipEventDestroy(g->ev0);
+    if (g->ev1) (void)hipEventDestroy(g->ev1);
+    if (g->stream) (void)hipStreamDestroy(g->stream);
+    if (g->h_meta) (void)hipHostFree(g->h_meta);
+    if (g->h_logits) (void)hipHostFree(g->h_logits);
+    if (g->h_small) (void)hipHostFree(g->h_small);
+    if (g->h_u) (void)hipHostFree(g->h_u);
+    if (g->arena) (void)hipFree(g->arena);
+    delete g;
+    return ZG_OK;
+}
+
+int zg_lm_load_tensor(zg_lm* g, const char* name, const float* data, size_t len) {
+    ZG_REQUIRE(g && name && data, ZG_ERR_ARG, "lm_load_tensor: bad argument");
+    ZG_HIP(hipSetDevice(g->device));
+    auto it = g->tensors.find(name);
+    ZG_REQUIRE(it != g->tensors.end(), ZG_ERR_ARG, "lm_load_tensor: the configuration has no tensor '%s'", name);
+    Tensor& t = it->second;
+    ZG_REQUIRE(len == t.rows * t.cols, ZG_ERR_SHAPE, "lm_load_tensor: '%s' has %zu elements, the configuration needs [%zu, %zu]", name, len, t.rows,
+               t.cols);
+    ZG_HIP(hipStreamSynchronize(g->stream));
+    if (!t.matrix) {
+        ZG_HIP(hipMemcpy(t.dev, data, len * sizeof(float), hipMemcpyHostToDevice));
+    } else {
+        std::vector<bf16_t> tmp(len);
+        auto rne = [](float x) {
+            uint32_t b;
+            memcpy(&b, &x, 4);
+            if ((b & 0x7F800000u) == 0x7F800000u) return (bf16_t)(b >> 16);  // inf / NaN keep their class
+            b += 0x7FFFu + ((b >> 16) & 1u);
+            return (bf16_t)(b >> 16);
+        };
+        if (t.transpose_heads > 0) {  // [heads * d][cols] -> [heads][cols][d]
+            const size_t Hh = t.transpose_heads, dd = t.rows / Hh, cc = t.cols;
+            for (size_t hh = 0; hh < Hh; ++hh)
+                for (size_t i = 0; i < dd; ++i)
+                    for (size_t c = 0; c < cc; ++c) tmp[(hh * cc + c) * dd + i] = rne(data[(hh * dd + i) * cc + c]);
+        } else {
+            for (size_t i = 0; i < len; ++i) tmp[i] = rne(data[i]);
+        }
+        ZG_HIP(hipMemcpy(t.dev, tmp.data(), len * sizeof(bf16_t), hipMemcpyHostToDevice));
+    }
+    t.loaded = true;
+    return ZG_OK;
+}
+
+int zg_lm_missing_tensors(zg_lm* g, size_t* count, char* names_out, size_t names_cap) {
+    ZG_REQUIRE(g && count, ZG_ERR_ARG, "lm_missing_tensors: bad argument");
+    size_t n = 0, off = 0;
+    if (names_out && names_cap) names_out[0] = 0;
+    for (auto& kv : g->tensors)
+        if (!kv.second.loaded) {
+            ++n;
+            if (names_out && off + kv.first.size() + 2 < names_cap) {
+                off += (size_t)snprintf(names_out + off, names_cap - off, "%s%s", off ? " " : "", kv.first.c_str());
+            }
+        }
+    *count = n;
+    return ZG_OK;
+}
+
+int zg_lm_init_random(zg_lm* g, uint64_t seed, float std_) {
+    ZG_REQUIRE(g && std_ > 0.0f, ZG_ERR_ARG, "lm_init_random: bad argument");
+    ZG_HIP(hipSetDevice(g->device));
+    uint64_t idx = 0;
+    for (auto& kv : g->tensors) {
+        Tensor& t = kv.second;
+        const size_t n = t.rows * t.cols;
+        fill_kernel<<<(unsigned)((n + 255) / 256), 256, 0, g->stream>>>(t.dev, n, seed * 0x9E3779B97F4A7C15ULL + (++idx) * 0xD1B54A32D192ED03ULL, t.init,
+                                                                        std_);
+        ZG_HIP(hipGetLastError());
+        t.loaded = true;
+    }
+    ZG_HIP(hipStreamSynchronize(g->stream));
+    return ZG_OK;
+}
+
+int zg_lm_seq_open(zg_lm* g, int* seq_out) {
+    ZG_REQUIRE(g && seq_out, ZG_ERR_ARG, "lm_seq_open: bad argument");
+    ZG_HIP(hipSetDevice(g->device));
+    int sidx = -1;
+    for (int i = 0; i < g->NS && sidx < 0; ++i)
+        if (!g->slots[i].open) sidx = i;
+    ZG_REQUIRE(sidx >= 0, ZG_ERR_SHAPE, "lm_seq_open: all %d state slots are in use", g->NS);
+    // a slot starts from zeros: no previous row for the token shift, an empty recurrent state
+    const size_t nsh = (size_t)g->n_passes * g->W;
+    zero_kernel<<<(unsigned)((nsh + 255) / 256), 256, 0, g->stream>>>(g->shift_state + (size_t)sidx * nsh, nsh);
+    ZG_HIP(hipGetLastError());
+    if (g->hgrn_floats) {
+        zero_kernel<<<(unsigned)((g->hgrn_floats + 255) / 256), 256, 0, g->stream>>>(g->hgrn_state + (size_t)sidx * g->hgrn_floats, g->hgrn_floats);
+        ZG_HIP(hipGetLastError());
+    }
+    Slot& sl = g->slots[sidx];
+    sl.open = true;
+    sl.len = 0;
+    sl.pages.clear();
+    *seq_out = sidx;
+    return ZG_OK;
+}
+
+int zg_lm_seq_close(zg_lm* g, int seq) {
+    ZG_REQUIRE(g && seq >= 0 && seq < g->NS && g->slots[seq].open, ZG_ERR_ARG, "lm_seq_close: sequence %d is not open", seq);
+    Slot& sl = g->slots[seq];
+    for (int p : sl.pages) g->free_pages.push_back(p);
+    sl.pages.clear();
+    sl.open = false;
+    sl.len = 0;
+    return ZG_OK;
+}
+
+int zg_lm_seq_len(zg_lm* g, int seq, size_t* len_out) {
+    ZG_REQUIRE(g && len_out && seq >= 0 && seq < g->NS && g->slots[seq].open, ZG_ERR_ARG, "lm_seq_len: sequence %d is not open", seq);
+    *len_out = g->slots[seq].len;
+    return ZG_OK;
+}
+
+int zg_lm_free_tokens(zg_lm* g, size_t* tokens_out) {
+    ZG_REQUIRE(g && tokens_out, ZG_ERR_ARG, "lm_free_tokens: bad argument");
+    *tokens_out = g->free_pages.size() * (size_t)g->P;
+    return ZG_OK;
+}
+
+int zg_lm_step(zg_lm* g, const zg_lm_entry* entries, size_t n_entries, float* logits_out, size_t logits_len) {
+    if (g) {
+        size_t missing = 0;
+        zg_lm_missing_tensors(g, &missing, nullptr, 0);
+        ZG_REQUIRE(missing == 0, ZG_ERR_NOT_INITIALIZED, "lm_step: %zu tensors of the configuration have not been loaded", missing);
+    }
+    return step_impl(g, entries, n_entries, logits_out, logits_len, nullptr);
+}
+
+int zg_lm_generate(zg_lm* g, const int32_t* prompts, size_t prompt_stride, const size_t* prompt_lens, size_t n_prompts, size_t n_new, float temp,
+                   uint64_t seed, int32_t* out_tokens, size_t out_len) {
+    ZG_REQUIRE(g && prompts && prompt_lens && out_tokens && n_prompts >= 1 && temp >= 0.0f, ZG_ERR_ARG, "lm_generate: bad argument");
+    ZG_REQUIRE(out_len >= n_prompts * n_new, ZG_ERR_SHAPE, "lm_generate: out_tokens needs %zu elements", n_prompts * n_new);
+    ZG_REQUIRE(n_prompts <= (size_t)g->logit_rows, ZG_ERR_UNSUPPORTED, "lm_generate: %zu prompts (at most %d at a time)", n_prompts, g->logit_rows);
+    size_t missing = 0;
+    zg_lm_missing_tensors(g, &missing, nullptr, 0);
+    ZG_REQUIRE(missing == 0, ZG_ERR_NOT_INITIALIZED, "lm_generate: %zu tensors of the configuration have not been loaded", missing);
+    for (size_t b = 0; b < n_prompts; ++b)
+        ZG_REQUIRE(prompt_lens[b] >= 1 && prompt_lens[b] <= prompt_stride, ZG_ERR_ARG, "lm_generate: prompt %zu has %zu tokens", b, prompt_lens[b]);
+    if (n_new == 0) return ZG_OK;
+    std::vector<int> seqs;
+    int status = ZG_OK;
+    for (size_t b = 0; b < n_prompts && status == ZG_OK; ++b) {
+        int sq = -1;
+        status = zg_lm_seq_open(g, &sq);
+        if (status == ZG_OK) seqs.push_back(sq);
+    }
+    std::vector<int32_t> cur(n_prompts), zero(n_prompts, 0), last(n_prompts);
+    const Sampler sm{temp, seed, cur.data()};
+    std::vector<zg_lm_entry> ent(n_prompts);
+    float decode_ms = 0.0f;
+    size_t decode_steps = 0;
+    for (size_t i = 0; i < n_new && status == ZG_OK; ++i) {
+        for (size_t b = 0; b < n_prompts; ++b) {
+            ent[b].seq = seqs[b];
+            if (i == 0) {  // the prompts, cut into portions by the step
+                ent[b].tokens = prompts + b * prompt_stride;
+                ent[b].n_tokens = prompt_lens[b];
+                last[b] = (int32_t)(prompt_lens[b] - 1);
+                ent[b].want = &last[b];
+            } else {
+                ent[b].tokens = &out_tokens[b * n_new + i - 1];
+                ent[b].n_tokens = 1;
+                ent[b].want = &zero[b];
+            }
+            ent[b].n_want = 1;
+        }
+        status = step_impl(g, ent.data(), n_prompts, nullptr, 0, &sm);
+        if (status != ZG_OK) break;
+        if (i > 0) {
+            decode_ms += g->last_step_ms;
+            ++decode_steps;
+        }
+        for (size_t b = 0; b < n_prompts; ++b) out_tokens[b * n_new + i] = cur[b];
+    }
+    g->last_decode_ms = decode_steps ? decode_ms / (float)decode_steps : 0.0f;
+    for (int sq : seqs) zg_lm_seq_close(g, sq);
+    return status;
+}
+
+int zg_lm_set_trace(zg_lm* g, float* trace_out, size_t trace_floats) {
+    ZG_REQUIRE(g, ZG_ERR_ARG, "lm_set_trace: bad argument");
+    g->trace = trace_out;
+    g->trace_floats = trace_out ? trace_floats : 0;
+    return ZG_OK;
+}
+
+int zg_lm_last_ms(zg_lm* g, float* step_ms, float* decode_ms_per_step) {
+    ZG_REQUIRE(g, ZG_ERR_ARG, "lm_last_ms: bad argument");
+    if (step_ms) *step_ms = g->last_step_ms;
+    if (decode_ms_per_step) *decode_ms_per_step = g->last_decode_ms;
+    return ZG_OK;
+}
+
+}  // extern "C"

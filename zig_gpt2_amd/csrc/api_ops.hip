@@ -11,34 +11,6 @@
 
 namespace zg {
 
-static thread_local char g_err[512] = "";
-
-int decode_paths_off() {
-    const char* e = getenv("ZGPT2_DECODE_PATHS_OFF");
-    return e ? atoi(e) : 0;
-}
-
-void set_error(const char* fmt, ...) {
-    va_list ap;
-    va_start(ap, fmt);
-    vsnprintf(g_err, sizeof(g_err), fmt, ap);
-    va_end(ap);
-}
-
-static thread_local char g_kernel[160] = "";
-void note_kernel(const char* fmt, ...) {
-    va_list ap;
-    va_start(ap, fmt);
-    vsnprintf(g_kernel, sizeof(g_kernel), fmt, ap);
-    va_end(ap);
-}
-
-int hip_fail(hipError_t e, const char* what, const char* file, int line) {
-    set_error("HIP error %d (%s) at %s:%d: %s", (int)e, hipGetErrorString(e), file, line, what);
-    (void)hipGetLastError();
-    return ZG_ERR_HIP;
-}
-
 Ctx& ctx() {
     static Ctx c;
     return c;
@@ -403,7 +375,6 @@ using namespace zg;
 
 extern "C" {
 
-const char* zg_last_error(void) { return zg::g_err; }
 
 static size_t env_mb(const char* name, size_t dflt) {
     if (const char* e = getenv(name)) {
@@ -622,11 +593,6 @@ int zg_debug_prefill_route(int force_kernel, int slices) {
 
 unsigned long long zg_debug_gemm_launches(void) { return gemm_mfma_launch_count(); }
 int zg_debug_gemm_stamps(unsigned long long* out, size_t n_words) { return gemm_debug_stamps(out, n_words); }
-int zg_debug_last_kernel(char* out, size_t n) {
-    if (!out || n == 0) return ZG_ERR_ARG;
-    snprintf(out, n, "%s", zg::g_kernel);
-    return ZG_OK;
-}
 
 int zg_f32_to_bf16(const float* src, uint16_t* dst_device, size_t len) {
     ZG_TRY(require_init());

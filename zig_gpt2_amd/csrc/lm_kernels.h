@@ -1,0 +1,114 @@
+// lm_kernels.h — launchers of the layered-model tier (api_lm.hip): a decoder stack whose layers are described by data (which
+// mixer, which feed-forward, which sizes), served for ragged batches of sequences that each own a state slot.
+//
+// Conventions shared by every launcher below
+//   * Activations are fp32 rows in device memory; weights are bf16 [out][in] row-major (K contiguous), vectors fp32.
+//   * A step carries M token rows (all entries of the batch back to back).  Per-row metadata lives in device arrays:
+//     row_pos (position of the token in its sequence), row_slot (state slot of its sequence), row_prev (row index of the token
+//     in front of it when that token is part of the same step, -1 when it is held by the slot's state).
+//   * `f32` selects true 32-bit products (fp32 MFMA / fp32 FMA) instead of bf16 x bf16 products with fp32 accumulation.
+//     Norms, softmax, gates, recurrent state, positions and the residual are fp32 in both modes.
+#pragma once
+#include "zg_common.h"
+
+namespace zg {
+namespace lm {
+
+// ------------------------------------------------------------------------------------------------ linear maps
+enum { ACT_NONE = 0, ACT_RELU2 = 1 };
+
+// C[m][n] = act( sum_k A[arow(m)][k] * B[n][k] )      for m < M, n < N
+//   arow(m) = a_rows ? a_rows[m] / a_div : m          (row gather: a token's row feeds each of its expert assignments)
+//   nz > 1: grid.z batches with element offsets a_zoff / b_zoff / c_zoff per z (one matrix per head)
+//   z_group != null: batch z reads the matrix B + z_group[z] * b_zoff instead (the expert an assignment was routed to)
+//   grp_off != null (n_groups > 0): rows [grp_off[e], grp_off[e + 1]) of A / C use the matrix B + e * b_zoff (rows sorted by
+//   expert); M is then the total row count, an upper bound for the tile list
+struct Linear {
+    const float* A = nullptr;
+    int lda = 0;
+    const int* a_rows = nullptr;
+    int a_div = 1;
+    const bf16_t* B = nullptr;
+    int ldb = 0;
+    float* C = nullptr;
+    int ldc = 0;
+    int M = 0, N = 0, K = 0;
+    int act = ACT_NONE;
+    int nz = 1;
+    long long a_zoff = 0, b_zoff = 0, c_zoff = 0;
+    const int* z_group = nullptr;
+    const int* grp_off = nullptr;
+    int n_groups = 0;
+};
+// Picks the row-vector kernel (few rows: decode) or the tiled matrix-core kernel (prompt portions).
+int launch_linear(const Linear& L, bool f32, hipStream_t s);
+constexpr int kGemvMaxRows = 8;
+
+// ------------------------------------------------------------------------------------------------ norms, embedding, shift
+// x[m] = table[ids[m]] (bf16 -> fp32); an id outside [0, vocab) raises *flag (pinned or device int) and yields a zero row.
+int launch_embed(const bf16_t* table, const int* ids, float* x, int M, int W, int vocab, int* flag, hipStream_t s);
+// RMS norm with a weight stored as an offset from one, then the token shift:
+//   h[m] = x[m] / rms(x[m]) * (1 + w);   out[m] = h[m] + (h[prev(m)] - h[m]) * mu
+// prev(m) = row_prev[m] when >= 0, else the row kept for the slot: shift_state[row_slot[m]] (zeros for a new sequence).
+// Rows listed in last_rows (the last token of every entry) also store their UNSHIFTED h into last_out[entry] — committed to
+// the slots' state by launch_commit_rows once the step has run, so that no row of this launch reads a state another row wrote.
+// mu == null: no shift (out = h).
+int launch_norm_shift(const float* x, const float* w, const float* mu, float eps, float* out, int M, int W, const int* row_prev,
+                      const int* row_slot, const float* shift_state, size_t slot_stride, const int* row_entry_if_last, float* last_out,
+                      hipStream_t s);
+// dst[slots[e]] = src[e] for every entry e; rows of `width` floats (dst rows slot_stride apart, src rows src_stride apart)
+int launch_commit_rows(float* dst, size_t slot_stride, const float* src, size_t src_stride, const int* slots, int n_entries, int width,
+                       int n_sets, size_t dst_set_stride, size_t src_set_stride, hipStream_t s);
+// x[m] += y[m] / rms(y[m]) * (1 + w)            (the norm behind a sublayer, then the residual sum)
+int launch_norm_add(float* x, const float* y, const float* w, float eps, int M, int W, hipStream_t s);
+// out[j] = x[rows[j]] / rms * (1 + w)            (the model's last norm on the rows whose logits are asked for)
+int launch_norm_gather(const float* x, const int* rows, const float* w, float eps, float* out, int n_rows, int W, hipStream_t s);
+// In place over `rows` rows of `width` floats with row stride ld: v / rms(v) * w  (a plain weight; per-head norms)
+int launch_norm_plain(float* v, int ld, int rows_per_m, int width, int M, const float* w, float eps, hipStream_t s);
+
+// ------------------------------------------------------------------------------------------------ gated linear recurrence (HGRN2)
+// proj rows are [q (H D) | f (H D) | v (H V)] as the fused projection left them.  Activates in place:
+//   q <- silu(q);   f <- low + (1 - low) * sigmoid(f + bias)
+int launch_hgrn2_gates(float* proj, int ld, int M, int HD, const float* bias, const float* low, hipStream_t s);
+// Per entry e (rows ent_start[e] .. + ent_len[e]) and head: S <- diag(f_t) S + (1 - f_t) v_t^T, o_t = S^T q_t, token by token,
+// S = state[ent_slot[e]] ([H][D][V] fp32) read at the start and written back at the end.  out rows [H V], row stride ldo.
+int launch_hgrn2_scan(const float* proj, int ld, float* out, int ldo, float* state, size_t slot_stride, const int* ent_start,
+                      const int* ent_len, const int* ent_slot, int n_entries, int H, int D, int V, hipStream_t s);
+
+// ------------------------------------------------------------------------------------------------ latent attention
+// Rotary table of one layer: freq[i] for the rot_dims / 2 pairs (YaRN blend applied on the host) and the amplitude factor.
+// proj rows: [dq (q_rank) | dkv latent (KR) | rotated key part (R)].  Writes cq[m] = norm(dq) * wq, and the token's cache row
+// (latent = norm(dkv latent) * wkv | rotary(key part)) at its position: cache row of (slot, pos) = page_table[slot][pos / P] * P + pos % P.
+struct Rotary {
+    const float* freq;  // [dims / 2]
+    int dims;           // rotated dimensions (the first `dims` of the part; the rest pass)
+    float amp;
+};
+int launch_latent_prep(const float* proj, int ld, int M, int q_rank, int KR, int R, const float* wq, const float* wkv, float eps, Rotary rot,
+                       const int* row_pos, const int* row_slot, const int* page_table, int max_pages, int page_tokens, float* cq,
+                       float* cache, hipStream_t s);
+// qa[m][h][KR ..] = rotary(q[m][h][D ..]) — the rotated query part moved behind the absorbed part (which a batched Linear wrote).
+int launch_q_rotary(const float* q, int ldq, float* qa, int ldqa, int M, int H, int D, int R, int KR, Rotary rot, const int* row_pos, hipStream_t s);
+// ctx[m][h][:KR] = sum_j softmax_j( scale * qa[m][h] . cacherow(j) ) latent(j) over the keys j <= row_pos[m] of the row's sequence.
+// ws: fp32 workspace for the partials of split key ranges (decode), ws_floats its size.
+int launch_latent_attention(const float* qa, float* ctx, int M, int H, int KR, int R, float scale, const int* row_pos, const int* row_slot,
+                            const int* page_table, int max_pages, int page_tokens, const float* cache, float* ws, size_t ws_floats, hipStream_t s);
+
+// ------------------------------------------------------------------------------------------------ mixture of experts
+// Per row: z = router . g (fp32), s = softmax(z), the `top` experts by s + correction (lowest index wins a tie), weights s.
+int launch_route(const float* g, int M, int W, const bf16_t* router, const float* correction, int E, int top, int* pick, float* weight,
+                 hipStream_t s);
+// Sort the M * top assignments by expert: grp_off[E + 1], sorted[p] = assignment at sorted position p, inv[a] = position of a.
+int launch_group(const int* pick, int n_assign, int E, int* grp_off, int* sorted, int* inv, hipStream_t s);
+// h[p][j] = silu(gu[p][j]) * gu[p][F + j]
+int launch_glu(const float* gu, float* h, int rows, int F, hipStream_t s);
+// y = sum_k weight[m][k] * yexp[inv ? inv[m top + k] : m top + k];   x[m] += y / rms(y) * (1 + w)
+int launch_moe_combine(float* x, const float* yexp, const int* inv, const float* weight, int top, const float* w, float eps, int M, int W,
+                       hipStream_t s);
+
+// ------------------------------------------------------------------------------------------------ sampling support
+// Per row: the maximum of its logits and the index of the first element that reaches it.
+int launch_row_argmax(const float* logits, int rows, int n, float* max_out, int* idx_out, hipStream_t s);
+
+}  // namespace lm
+}  // namespace zg

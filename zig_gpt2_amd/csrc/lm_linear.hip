@@ -1,0 +1,347 @@
+// lm_linear.hip — the linear maps of the layered-model tier: C = act(A B^T) with fp32 activation rows A and bf16 weights B.
+//
+// Two kernels behind one launcher:
+//   * lm_gemv_kernel   up to 8 rows (decode steps): a wave owns two weight rows, its lanes split K in 16-byte pieces, the
+//                      activation rows come straight from the cache hierarchy, sums are fp32 FMAs in both precision modes.
+//   * lm_gemm_kernel   prompt portions: 64 x 64 or 128 x 128 tiles on the matrix cores, four waves in a 2 x 2 arrangement of
+//                      32 x 32 MFMA tiles.  bf16 mode rounds the activations to bf16 on their way into the LDS and multiplies with
+//                      v_mfma_f32_32x32x16_bf16 (fp32 accumulation); 32-bit mode widens the weights and multiplies with
+//                      v_mfma_f32_32x32x2_f32.  Any M, N, K: tiles are zero-filled at the edges.
+// Both understand the same addressing: a row gather for A, one matrix per grid.z batch (heads), a matrix chosen per batch by
+// an index array (the expert of an assignment), and row groups sorted by expert with their offsets in device memory.
+#include <type_traits>
+
+#include "lm_kernels.h"
+
+namespace zg {
+namespace lm {
+
+namespace {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+
+struct LinArgs {
+    const float* A;
+    const bf16_t* B;
+    float* C;
+    const int* a_rows;
+    const int* z_group;
+    const int* grp_off;
+    long long a_zoff, b_zoff, c_zoff;
+    int lda, ldb, ldc;
+    int M, N, K;
+    int a_div, act, n_groups;
+    int a_vec, b_vec;  // 16-byte loads allowed (alignment of base, leading dimension and batch offsets)
+};
+
+__device__ __forceinline__ float apply_act(float v, int act) {
+    if (act == ACT_RELU2) {
+        v = fmaxf(v, 0.0f);
+        v = v * v;
+    }
+    return v;
+}
+
+// eight consecutive weights of row `w` from column k, zero beyond K
+__device__ __forceinline__ void load_w8(const bf16_t* w, int k, int K, bool vec, float out[8]) {
+    if (vec && k + 8 <= K) {
+        const u32x4 p = *reinterpret_cast<const u32x4*>(w + k);
+        out[0] = bf16_lo(p.x); out[1] = bf16_hi(p.x); out[2] = bf16_lo(p.y); out[3] = bf16_hi(p.y);
+        out[4] = bf16_lo(p.z); out[5] = bf16_hi(p.z); out[6] = bf16_lo(p.w); out[7] = bf16_hi(p.w);
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) out[i] = (k + i < K) ? __uint_as_float((uint32_t)w[k + i] << 16) : 0.0f;
+    }
+}
+
+__device__ __forceinline__ f32x4 load_a4(const float* a, int k, int K, bool vec) {
+    if (a == nullptr) return f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    if (vec && k + 4 <= K) return *reinterpret_cast<const f32x4*>(a + k);
+    f32x4 r;
+    r.x = (k + 0 < K) ? a[k + 0] : 0.0f;
+    r.y = (k + 1 < K) ? a[k + 1] : 0.0f;
+    r.z = (k + 2 < K) ? a[k + 2] : 0.0f;
+    r.w = (k + 3 < K) ? a[k + 3] : 0.0f;
+    return r;
+}
+
+// ------------------------------------------------------------------------------------------------ few rows
+template <int MR>
+__global__ __launch_bounds__(256) void lm_gemv_kernel(const LinArgs p) {
+    const int z = blockIdx.z, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int n0 = blockIdx.x * 8 + wave * 2;
+    if (n0 >= p.N) return;
+    const bf16_t* B = p.B + (long long)(p.z_group ? p.z_group[z] : z) * p.b_zoff;
+    const float* A = p.A + (long long)z * p.a_zoff;
+    float* C = p.C + (long long)z * p.c_zoff;
+    const float* arow[MR];
+#pragma unroll
+    for (int m = 0; m < MR; ++m) {
+        arow[m] = nullptr;
+        if (m < p.M) {
+            const int rid = p.z_group ? z * p.M + m : m;
+            const int src = (p.a_rows ? p.a_rows[rid] : rid) / p.a_div;
+            arow[m] = A + (long long)src * p.lda;
+        }
+    }
+    const bool two = n0 + 1 < p.N;
+    const bf16_t* w0 = B + (long long)n0 * p.ldb;
+    const bf16_t* w1 = B + (long long)(two ? n0 + 1 : n0) * p.ldb;
+    float acc0[MR], acc1[MR];
+#pragma unroll
+    for (int m = 0; m < MR; ++m) acc0[m] = acc1[m] = 0.0f;
+    for (int k = lane * 8; k < p.K; k += 512) {
+        float wa[8], wb[8];
+        load_w8(w0, k, p.K, p.b_vec, wa);
+        load_w8(w1, k, p.K, p.b_vec, wb);
+#pragma unroll
+        for (int m = 0; m < MR; ++m) {
+            const f32x4 a0 = load_a4(arow[m], k, p.K, p.a_vec), a1 = load_a4(arow[m], k + 4, p.K, p.a_vec);
+            float s0 = acc0[m], s1 = acc1[m];
+            s0 = fmaf(a0.x, wa[0], s0); s1 = fmaf(a0.x, wb[0], s1);
+            s0 = fmaf(a0.y, wa[1], s0); s1 = fmaf(a0.y, wb[1], s1);
+            s0 = fmaf(a0.z, wa[2], s0); s1 = fmaf(a0.z, wb[2], s1);
+            s0 = fmaf(a0.w, wa[3], s0); s1 = fmaf(a0.w, wb[3], s1);
+            s0 = fmaf(a1.x, wa[4], s0); s1 = fmaf(a1.x, wb[4], s1);
+            s0 = fmaf(a1.y, wa[5], s0); s1 = fmaf(a1.y, wb[5], s1);
+            s0 = fmaf(a1.z, wa[6], s0); s1 = fmaf(a1.z, wb[6], s1);
+            s0 = fmaf(a1.w, wa[7], s0); s1 = fmaf(a1.w, wb[7], s1);
+            acc0[m] = s0;
+            acc1[m] = s1;
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < MR; ++m) {
+        const float s0 = wave_allsum(acc0[m]), s1 = wave_allsum(acc1[m]);
+        if (lane == 0 && m < p.M) {
+            C[(long long)m * p.ldc + n0] = apply_act(s0, p.act);
+            if (two) C[(long long)m * p.ldc + n0 + 1] = apply_act(s1, p.act);
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------ matrix cores
+template <bool F32>
+struct Tile {
+    static constexpr int BK = F32 ? 16 : 32;
+    static constexpr int LDS_K = F32 ? 17 : 40;  // row stride in elements: conflict-free fragment reads
+    typedef typename std::conditional<F32, float, bf16_t>::type elem;
+};
+
+template <bool F32, int WT>  // WT x WT MFMA tiles of 32 x 32 per wave; workgroup tile = 64 WT squared
+__global__ __launch_bounds__(256) void lm_gemm_kernel(const LinArgs p) {
+    typedef Tile<F32> T;
+    typedef typename T::elem elem;
+    constexpr int BM = 64 * WT, BN = 64 * WT, BK = T::BK, LK = T::LDS_K;
+    __shared__ __attribute__((aligned(16))) elem As[BM * LK];
+    __shared__ __attribute__((aligned(16))) elem Bs[BN * LK];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wy = wave >> 1, wx = wave & 1;
+    const int z = blockIdx.z;
+    const bf16_t* B = p.B;
+    int m0, m_end;
+    if (p.grp_off) {  // find the row group this tile belongs to
+        int tile = blockIdx.y, e = 0, lo = 0, hi = 0;
+        for (; e < p.n_groups; ++e) {
+            lo = p.grp_off[e];
+            hi = p.grp_off[e + 1];
+            const int nt = (hi - lo + BM - 1) / BM;
+            if (tile < nt) break;
+            tile -= nt;
+        }
+        if (e >= p.n_groups) return;
+        m0 = lo + tile * BM;
+        m_end = hi;
+        B += (long long)e * p.b_zoff;
+    } else {
+        m0 = blockIdx.y * BM;
+        m_end = p.M;
+        B += (long long)(p.z_group ? p.z_group[z] : z) * p.b_zoff;
+    }
+    const float* A = p.A + (long long)z * p.a_zoff;
+    float* C = p.C + (long long)z * p.c_zoff;
+    const int n0 = blockIdx.x * BN;
+
+    // global -> register assignment of this thread (fixed over the K loop)
+    constexpr int A_VEC_PER_ROW = BK / 4;                 // float4 per A row of the tile
+    constexpr int A_LOADS = BM * A_VEC_PER_ROW / 256;     // per thread
+    constexpr int B_VEC_PER_ROW = BK / 8;                 // 8 bf16 per vector
+    constexpr int B_LOADS = (BN * B_VEC_PER_ROW + 255) / 256;
+    const float* a_src[A_LOADS];
+    int a_r[A_LOADS], a_k[A_LOADS];
+#pragma unroll
+    for (int j = 0; j < A_LOADS; ++j) {
+        const int v = tid + 256 * j;
+        a_r[j] = v / A_VEC_PER_ROW;
+        a_k[j] = (v % A_VEC_PER_ROW) * 4;
+        const int m = m0 + a_r[j];
+        a_src[j] = nullptr;
+        if (m < m_end) {
+            const int rid = p.z_group ? z * p.M + m : m;
+            const int src = (p.a_rows ? p.a_rows[rid] : rid) / p.a_div;
+            a_src[j] = A + (long long)src * p.lda;
+        }
+    }
+    const bf16_t* b_src[B_LOADS];
+    int b_r[B_LOADS], b_k[B_LOADS];
+#pragma unroll
+    for (int j = 0; j < B_LOADS; ++j) {
+        const int v = tid + 256 * j;
+        b_r[j] = v / B_VEC_PER_ROW;
+        b_k[j] = (v % B_VEC_PER_ROW) * 8;
+        const int n = n0 + b_r[j];
+        b_src[j] = (b_r[j] < BN && n < p.N) ? B + (long long)n * p.ldb : nullptr;
+    }
+
+    f32x16 acc[WT][WT];
+#pragma unroll
+    for (int i = 0; i < WT; ++i)
+#pragma unroll
+        for (int j = 0; j < WT; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+    f32x4 a_reg[A_LOADS];
+    float b_reg[B_LOADS][8];
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int j = 0; j < A_LOADS; ++j) a_reg[j] = load_a4(a_src[j], k0 + a_k[j], p.K, p.a_vec);
+#pragma unroll
+        for (int j = 0; j < B_LOADS; ++j) {
+            if (b_src[j]) {
+                load_w8(b_src[j], k0 + b_k[j], p.K, p.b_vec, b_reg[j]);
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) b_reg[j][i] = 0.0f;
+            }
+        }
+    };
+    auto stash = [&]() {
+#pragma unroll
+        for (int j = 0; j < A_LOADS; ++j) {
+            elem* d = &As[a_r[j] * LK + a_k[j]];
+            if constexpr (F32) {
+                d[0] = a_reg[j].x; d[1] = a_reg[j].y; d[2] = a_reg[j].z; d[3] = a_reg[j].w;
+            } else {
+                u32x2 pk;
+                pk.x = cvt_pk_bf16(a_reg[j].x, a_reg[j].y);
+                pk.y = cvt_pk_bf16(a_reg[j].z, a_reg[j].w);
+                *reinterpret_cast<u32x2*>(d) = pk;
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < B_LOADS; ++j) {
+            if (b_r[j] < BN) {
+                elem* d = &Bs[b_r[j] * LK + b_k[j]];
+                if constexpr (F32) {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) d[i] = b_reg[j][i];
+                } else {
+                    u32x4 pk;  // the values are bf16 already: the conversion is exact
+                    pk.x = cvt_pk_bf16(b_reg[j][0], b_reg[j][1]);
+                    pk.y = cvt_pk_bf16(b_reg[j][2], b_reg[j][3]);
+                    pk.z = cvt_pk_bf16(b_reg[j][4], b_reg[j][5]);
+                    pk.w = cvt_pk_bf16(b_reg[j][6], b_reg[j][7]);
+                    *reinterpret_cast<u32x4*>(d) = pk;
+                }
+            }
+        }
+    };
+
+    fetch(0);
+    for (int k0 = 0; k0 < p.K; k0 += BK) {
+        __syncthreads();  // the previous step's fragment reads are done
+        stash();
+        __syncthreads();
+        if (k0 + BK < p.K) fetch(k0 + BK);  // in flight beside the MFMAs
+        const int r = lane & 31, kh = lane >> 5;
+        if constexpr (F32) {
+#pragma unroll
+            for (int kk = 0; kk < BK; kk += 2) {
+                float af[WT], bf[WT];
+#pragma unroll
+                for (int i = 0; i < WT; ++i) af[i] = As[((wy * WT + i) * 32 + r) * LK + kk + kh];
+#pragma unroll
+                for (int j = 0; j < WT; ++j) bf[j] = Bs[((wx * WT + j) * 32 + r) * LK + kk + kh];
+#pragma unroll
+                for (int i = 0; i < WT; ++i)
+#pragma unroll
+                    for (int j = 0; j < WT; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i], bf[j], acc[i][j], 0, 0, 0);
+            }
+        } else {
+#pragma unroll
+            for (int kk = 0; kk < BK; kk += 16) {
+                bf16x8 af[WT], bf[WT];
+#pragma unroll
+                for (int i = 0; i < WT; ++i)
+                    af[i] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(&As[((wy * WT + i) * 32 + r) * LK + kk + kh * 8]));
+#pragma unroll
+                for (int j = 0; j < WT; ++j)
+                    bf[j] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(&Bs[((wx * WT + j) * 32 + r) * LK + kk + kh * 8]));
+#pragma unroll
+                for (int i = 0; i < WT; ++i)
+#pragma unroll
+                    for (int j = 0; j < WT; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bf[j], acc[i][j], 0, 0, 0);
+            }
+        }
+    }
+
+    // accumulator element e of a 32 x 32 tile: row 8 (e / 4) + 4 (lane / 32) + e % 4, column lane % 32
+#pragma unroll
+    for (int i = 0; i < WT; ++i)
+#pragma unroll
+        for (int j = 0; j < WT; ++j) {
+            const int n = n0 + (wx * WT + j) * 32 + (lane & 31);
+            if (n >= p.N) continue;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int m = m0 + (wy * WT + i) * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+                if (m < m_end) C[(long long)m * p.ldc + n] = apply_act(acc[i][j][e], p.act);
+            }
+        }
+}
+
+}  // namespace
+
+int launch_linear(const Linear& L, bool f32, hipStream_t s) {
+    if (L.M <= 0 || L.N <= 0 || L.nz <= 0) return ZG_OK;
+    ZG_REQUIRE(L.K > 0 && L.A && L.B && L.C, ZG_ERR_ARG, "linear: empty operand");
+    ZG_REQUIRE(L.a_div >= 1, ZG_ERR_ARG, "linear: a_div %d", L.a_div);
+    LinArgs p;
+    p.A = L.A; p.B = L.B; p.C = L.C; p.a_rows = L.a_rows; p.z_group = L.z_group; p.grp_off = L.grp_off;
+    p.a_zoff = L.a_zoff; p.b_zoff = L.b_zoff; p.c_zoff = L.c_zoff;
+    p.lda = L.lda; p.ldb = L.ldb; p.ldc = L.ldc; p.M = L.M; p.N = L.N; p.K = L.K;
+    p.a_div = L.a_div; p.act = L.act; p.n_groups = L.grp_off ? L.n_groups : 0;
+    p.a_vec = ((reinterpret_cast<uintptr_t>(L.A) & 15) == 0 && L.lda % 4 == 0 && L.a_zoff % 4 == 0) ? 1 : 0;
+    p.b_vec = ((reinterpret_cast<uintptr_t>(L.B) & 15) == 0 && L.ldb % 8 == 0 && L.b_zoff % 8 == 0) ? 1 : 0;
+    if (!L.grp_off && L.M <= kGemvMaxRows) {
+        const dim3 grid((L.N + 7) / 8, 1, L.nz);
+        if (L.M == 1) lm_gemv_kernel<1><<<grid, 256, 0, s>>>(p);
+        else if (L.M == 2) lm_gemv_kernel<2><<<grid, 256, 0, s>>>(p);
+        else if (L.M <= 4) lm_gemv_kernel<4><<<grid, 256, 0, s>>>(p);
+        else lm_gemv_kernel<8><<<grid, 256, 0, s>>>(p);
+        note_kernel("lm_gemv_kernel<%d>", L.M == 1 ? 1 : L.M == 2 ? 2 : L.M <= 4 ? 4 : 8);
+        ZG_HIP(hipGetLastError());
+        return ZG_OK;
+    }
+    ZG_REQUIRE(!(L.z_group && L.grp_off), ZG_ERR_ARG, "linear: a matrix per batch and row groups exclude each other");
+    auto tiles = [&](int b) { return (long long)((L.M + b - 1) / b + (L.grp_off ? L.n_groups : 0)) * ((L.N + b - 1) / b) * L.nz; };
+    const bool big = tiles(128) >= 512;
+    const int b = big ? 128 : 64;
+    const dim3 grid((L.N + b - 1) / b, (L.M + b - 1) / b + (L.grp_off ? L.n_groups : 0), L.nz);
+    ZG_REQUIRE(grid.y <= 65535 && grid.z <= 65535, ZG_ERR_UNSUPPORTED, "linear: %d rows in %d batches exceed the grid", L.M, L.nz);
+    if (f32) {
+        if (big) lm_gemm_kernel<true, 2><<<grid, 256, 0, s>>>(p);
+        else lm_gemm_kernel<true, 1><<<grid, 256, 0, s>>>(p);
+    } else {
+        if (big) lm_gemm_kernel<false, 2><<<grid, 256, 0, s>>>(p);
+        else lm_gemm_kernel<false, 1><<<grid, 256, 0, s>>>(p);
+    }
+    note_kernel("lm_gemm_kernel<%s, %d>", f32 ? "true" : "false", big ? 2 : 1);
+    ZG_HIP(hipGetLastError());
+    return ZG_OK;
+}
+
+}  // namespace lm
+}  // namespace zg

@@ -1,0 +1,177 @@
+// lm_moe.hip — routing of the mixture-of-experts feed-forward of the layered-model tier: router scores and the choice of experts
+// (fp32), the sort of a step's assignments by expert for the grouped matrix products, the gated activation, and the weighted
+// sum of the chosen experts' outputs fused with the norm and the residual sum behind the sublayer.
+#include <math.h>
+
+#include "lm_kernels.h"
+
+namespace zg {
+namespace lm {
+
+namespace {
+
+constexpr int kMaxExperts = 256;  // four per lane of the routing wave
+
+__device__ __forceinline__ float block_allsum(float v, float* s_red) {
+    v = wave_allsum(v);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+    __syncthreads();
+    if (lane == 0) s_red[wave] = v;
+    __syncthreads();
+    float t = 0.0f;
+    for (int w = 0; w < nw; ++w) t += s_red[w];
+    return t;
+}
+
+// one wave per row; lane l scores the experts l, l + 64, l + 128, l + 192
+__global__ __launch_bounds__(256) void route_kernel(const float* g, int M, int W, const bf16_t* router, const float* correction, int E, int top,
+                                                    int* pick, float* weight) {
+    const int m = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    if (m >= M) return;
+    const float* row = g + (size_t)m * W;
+    float z[4], sc[4], ch[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int e = lane + 64 * i;
+        z[i] = -INFINITY;
+        if (e < E) {
+            const bf16_t* wr = router + (size_t)e * W;
+            float a = 0.0f;
+            for (int k = 0; k < W; ++k) a = fmaf(row[k], __uint_as_float((uint32_t)wr[k] << 16), a);
+            z[i] = a;
+        }
+    }
+    const float mx = wave_allmax(fmaxf(fmaxf(z[0], z[1]), fmaxf(z[2], z[3])));
+    float sum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        sc[i] = expf(z[i] - mx);  // 0 for the experts that do not exist
+        sum += sc[i];
+    }
+    sum = wave_allsum(sum);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int e = lane + 64 * i;
+        sc[i] = sc[i] / sum;
+        ch[i] = e < E ? sc[i] + correction[e] : -INFINITY;
+    }
+    for (int k = 0; k < top; ++k) {
+        float best = -INFINITY;
+        int bi = 0x7fffffff;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if (ch[i] > best) {  // ascending expert index per lane: the first maximum stays
+                best = ch[i];
+                bi = lane + 64 * i;
+            }
+        const float wbest = wave_allmax(best);
+        int cand = (best == wbest) ? bi : 0x7fffffff;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) cand = min(cand, __shfl_xor(cand, off, 64));
+        if (cand == 0x7fffffff) cand = 0;  // nothing left to choose from (NaN scores): keep the indices in range
+        if ((cand & 63) == lane) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if ((cand >> 6) == i) {
+                    pick[(size_t)m * top + k] = cand;
+                    weight[(size_t)m * top + k] = sc[i];
+                    ch[i] = -INFINITY;
+                }
+        }
+    }
+}
+
+// one workgroup: histogram, offsets, placement.  The order inside a group is arbitrary: every row of a grouped product is
+// computed independently of its neighbours, so the results do not depend on it.
+__global__ __launch_bounds__(1024) void group_kernel(const int* pick, int n_assign, int E, int* grp_off, int* sorted, int* inv) {
+    __shared__ int s_cnt[kMaxExperts], s_off[kMaxExperts + 1], s_cur[kMaxExperts];
+    for (int e = threadIdx.x; e < E; e += blockDim.x) s_cnt[e] = s_cur[e] = 0;
+    __syncthreads();
+    for (int a = threadIdx.x; a < n_assign; a += blockDim.x) atomicAdd(&s_cnt[pick[a]], 1);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int o = 0;
+        for (int e = 0; e < E; ++e) {
+            s_off[e] = o;
+            o += s_cnt[e];
+        }
+        s_off[E] = o;
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e <= E; e += blockDim.x) grp_off[e] = s_off[e];
+    for (int a = threadIdx.x; a < n_assign; a += blockDim.x) {
+        const int e = pick[a];
+        const int p = s_off[e] + atomicAdd(&s_cur[e], 1);
+        sorted[p] = a;
+        inv[a] = p;
+    }
+}
+
+__global__ __launch_bounds__(256) void glu_kernel(const float* gu, float* h, size_t n, int F) {
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= n) return;
+    const size_t r = idx / F;
+    const int j = (int)(idx % F);
+    const float a = gu[r * 2 * F + j], b = gu[r * 2 * F + F + j];
+    h[idx] = a / (1.0f + expf(-a)) * b;
+}
+
+__global__ __launch_bounds__(256) void moe_combine_kernel(float* x, const float* yexp, const int* inv, const float* weight, int top, const float* w,
+                                                          float eps, int W) {
+    __shared__ float s_red[8];
+    const int m = blockIdx.x;
+    auto mix = [&](int i) {
+        float y = 0.0f;
+        for (int k = 0; k < top; ++k) {
+            const int a = m * top + k;
+            y = fmaf(weight[a], yexp[(size_t)(inv ? inv[a] : a) * W + i], y);
+        }
+        return y;
+    };
+    float ss = 0.0f;
+    for (int i = threadIdx.x; i < W; i += blockDim.x) {
+        const float y = mix(i);
+        ss = fmaf(y, y, ss);
+    }
+    ss = block_allsum(ss, s_red);
+    const float r = 1.0f / sqrtf(ss / (float)W + eps);
+    for (int i = threadIdx.x; i < W; i += blockDim.x) x[(size_t)m * W + i] += mix(i) * r * (1.0f + w[i]);
+}
+
+}  // namespace
+
+int launch_route(const float* g, int M, int W, const bf16_t* router, const float* correction, int E, int top, int* pick, float* weight,
+                 hipStream_t s) {
+    if (M <= 0) return ZG_OK;
+    ZG_REQUIRE(E >= 1 && E <= kMaxExperts && top >= 1 && top <= E, ZG_ERR_UNSUPPORTED, "router: %d experts, %d chosen (at most %d experts)", E, top,
+               kMaxExperts);
+    route_kernel<<<(M + 3) / 4, 256, 0, s>>>(g, M, W, router, correction, E, top, pick, weight);
+    ZG_HIP(hipGetLastError());
+    return ZG_OK;
+}
+
+int launch_group(const int* pick, int n_assign, int E, int* grp_off, int* sorted, int* inv, hipStream_t s) {
+    ZG_REQUIRE(E >= 1 && E <= kMaxExperts, ZG_ERR_UNSUPPORTED, "router: %d experts (at most %d)", E, kMaxExperts);
+    group_kernel<<<1, 1024, 0, s>>>(pick, n_assign, E, grp_off, sorted, inv);
+    ZG_HIP(hipGetLastError());
+    return ZG_OK;
+}
+
+int launch_glu(const float* gu, float* h, int rows, int F, hipStream_t s) {
+    const size_t n = (size_t)rows * F;
+    if (n == 0) return ZG_OK;
+    glu_kernel<<<(unsigned)((n + 255) / 256), 256, 0, s>>>(gu, h, n, F);
+    ZG_HIP(hipGetLastError());
+    return ZG_OK;
+}
+
+int launch_moe_combine(float* x, const float* yexp, const int* inv, const float* weight, int top, const float* w, float eps, int M, int W,
+                       hipStream_t s) {
+    if (M <= 0) return ZG_OK;
+    moe_combine_kernel<<<M, 256, 0, s>>>(x, yexp, inv, weight, top, w, eps, W);
+    ZG_HIP(hipGetLastError());
+    return ZG_OK;
+}
+
+}  // namespace lm
+}  // namespace zg

@@ -1,0 +1,286 @@
+"""Layered language models over the C ABI's layered-model tier (zg_lm_* of include/zgpt2.h).
+
+A model of this family is DATA: config.json lists the layers — which token mixer, which feed-forward, their sizes — and the
+library runs whatever list it is given.  This module turns a checkpoint's config.json into the library's layer descriptors
+(`LMConfig`), loads tensors by their checkpoint names, and wraps the handle (`LayeredLM`): sequences are opened, stepped with
+any number of tokens at a time (several sequences per step), and closed; `generate` runs prompts through the same step with
+the library's greedy / sampling head.
+
+config.json of the Tokosun design (the only architecture of the family so far; zig_gpt2_amd/models.py maps names to classes):
+  vocab, width, norm.eps, layers[i] = {type: "hgrn2" | "latent_attention", mixer: {...sizes...}, mlp: null | {kind: "dense", ff}
+  | {kind: "moe", expert: {ff}, router: {experts, top}}}, loop: null | {start, stop, times}.
+"""
+import ctypes as C
+import json
+import os
+from dataclasses import dataclass, field
+from typing import List, Optional
+
+import numpy as np
+
+from . import _lib
+from ._lib import check_lm as check
+
+MIXERS = {"hgrn2": _lib.LM_MIX_HGRN2, "latent_attention": _lib.LM_MIX_LATENT_ATTENTION}
+
+
+@dataclass
+class LayerSpec:
+    """One entry of config['layers'], flattened into the fields of zg_lm_layer."""
+
+    mixer: str
+    heads: int
+    dim: int
+    vdim: int
+    rot_dim: int = 0
+    kv_rank: int = 0
+    q_rank: int = 0
+    scale: float = 1.0
+    rot_dims: int = 0
+    rot_base: float = 10000.0
+    rot_scaling: Optional[dict] = None  # {factor, original, fast, slow}
+    ff: str = "none"  # none | dense | moe
+    ff_width: int = 0
+    experts: int = 0
+    top: int = 0
+
+    @classmethod
+    def from_json(cls, entry):
+        kind, m = entry["type"], entry["mixer"]
+        if kind not in MIXERS:
+            raise ValueError(f"unknown mixer type {kind!r} (known: {sorted(MIXERS)})")
+        kw = dict(mixer=kind, heads=int(m["heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]))
+        if kind == "latent_attention":
+            rot = m.get("rot") or {}
+            kw.update(rot_dim=int(m["rot_dim"]), kv_rank=int(m["kv_rank"]), q_rank=int(m["q_rank"]), scale=float(m["scale"]),
+                      rot_dims=int(rot.get("dims", m["rot_dim"])), rot_base=float(rot.get("base", 10000.0)),
+                      rot_scaling=dict(rot["scaling"]) if rot.get("scaling") else None)
+        mlp = entry.get("mlp")
+        if mlp:
+            if mlp["kind"] == "dense":
+                kw.update(ff="dense", ff_width=int(mlp["ff"]))
+            elif mlp["kind"] == "moe":
+                kw.update(ff="moe", ff_width=int(mlp["expert"]["ff"]), experts=int(mlp["router"]["experts"]), top=int(mlp["router"]["top"]))
+            else:
+                raise ValueError(f"unknown feed-forward kind {mlp['kind']!r}")
+        return cls(**kw)
+
+    def to_json(self):
+        mixer = {"heads": self.heads, "dim": self.dim, "vdim": self.vdim}
+        if self.mixer == "latent_attention":
+            rot = {"base": self.rot_base, "dims": self.rot_dims}
+            if self.rot_scaling:
+                rot["scaling"] = dict(self.rot_scaling)
+            mixer.update(rot_dim=self.rot_dim, kv_rank=self.kv_rank, q_rank=self.q_rank, scale=self.scale, rot=rot)
+        mlp = None
+        if self.ff == "dense":
+            mlp = {"kind": "dense", "ff": self.ff_width}
+        elif self.ff == "moe":
+            mlp = {"kind": "moe", "expert": {"ff": self.ff_width}, "router": {"experts": self.experts, "top": self.top}}
+        return {"type": self.mixer, "mixer": mixer, "mlp": mlp}
+
+    def to_c(self):
+        sc = self.rot_scaling or {}
+        return _lib.LmLayer(MIXERS[self.mixer], self.heads, self.dim, self.vdim, self.rot_dim, self.kv_rank, self.q_rank, self.scale, self.rot_dims,
+                            self.rot_base, 1 if self.rot_scaling else 0, float(sc.get("factor", 1.0)), float(sc.get("original", 1.0)),
+                            float(sc.get("fast", 1.0)), float(sc.get("slow", 1.0)),
+                            {"none": _lib.LM_FF_NONE, "dense": _lib.LM_FF_DENSE, "moe": _lib.LM_FF_MOE}[self.ff], self.ff_width, self.experts,
+                            self.top)
+
+    def tensor_shapes(self, prefix, width):
+        """{checkpoint tensor name: shape} of this layer."""
+        H, D, V, W = self.heads, self.dim, self.vdim, width
+        t = {prefix + "norm1": (W,), prefix + "norm1b": (W,), prefix + "shift": (W,)}
+        m = prefix + "mix."
+        if self.mixer == "hgrn2":
+            t.update({m + "q": (H * D, W), m + "f": (H * D, W), m + "f.b": (H * D,), m + "lower": (H * D,), m + "v": (H * V, W), m + "norm": (V,),
+                      m + "o": (W, H * V)})
+        else:
+            R, KR, QR = self.rot_dim, self.kv_rank, self.q_rank
+            t.update({m + "dq": (QR, W), m + "dq.norm": (QR,), m + "uq": (H * (D + R), QR), m + "dkv": (KR + R, W), m + "dkv.norm": (KR,),
+                      m + "uk": (H * D, KR), m + "uv": (H * V, KR), m + "o": (W, H * V)})
+        f = prefix + "mlp."
+        if self.ff != "none":
+            t.update({prefix + "norm2": (W,), prefix + "norm2b": (W,)})
+        if self.ff == "dense":
+            t.update({f + "up": (self.ff_width, W), f + "down": (W, self.ff_width)})
+        elif self.ff == "moe":
+            for e in range(self.experts):
+                t.update({f"{f}e{e}.gate": (self.ff_width, W), f"{f}e{e}.up": (self.ff_width, W), f"{f}e{e}.down": (W, self.ff_width)})
+            t.update({f + "router": (self.experts, W), f + "correction": (self.experts,)})
+        return t
+
+
+@dataclass
+class LMConfig:
+    vocab: int
+    width: int
+    layers: List[LayerSpec]
+    norm_eps: float = 1e-6
+    loop: Optional[dict] = None  # {start, stop, times}
+    architecture: str = "Tokosun"
+    extra: dict = field(default_factory=dict)
+
+    @classmethod
+    def from_json(cls, cfg):
+        return cls(vocab=int(cfg["vocab"]), width=int(cfg["width"]), layers=[LayerSpec.from_json(e) for e in cfg["layers"]],
+                   norm_eps=float(cfg["norm"]["eps"]), loop=dict(cfg["loop"]) if cfg.get("loop") else None,
+                   architecture=cfg.get("architecture", "Tokosun"))
+
+    @classmethod
+    def from_dir(cls, path):
+        with open(os.path.join(path, "config.json")) as f:
+            return cls.from_json(json.load(f))
+
+    def to_json(self):
+        return {"architecture": self.architecture, "vocab": self.vocab, "width": self.width, "norm": {"eps": self.norm_eps},
+                "layers": [l.to_json() for l in self.layers], "loop": dict(self.loop) if self.loop else None}
+
+    def passes(self):
+        """Layer index of every pass, in execution order."""
+        n = len(self.layers)
+        if not self.loop or int(self.loop["times"]) <= 1:
+            return list(range(n))
+        a, b, k = int(self.loop["start"]), int(self.loop["stop"]), int(self.loop["times"])
+        return list(range(a)) + list(range(a, b)) * k + list(range(b, n))
+
+    def tensor_shapes(self):
+        t = {"embed": (self.vocab, self.width), "head": (self.vocab, self.width), "final.norm": (self.width,)}
+        for i, l in enumerate(self.layers):
+            t.update(l.tensor_shapes(f"l{i}.", self.width))
+        return t
+
+
+class LayeredLM:
+    """A handle of the layered-model tier: weights, state slots, the step function and generation."""
+
+    def __init__(self, config: LMConfig, dtype="bfloat16", max_tokens=4096, max_seqs=8, max_step_tokens=0, page_tokens=0, device=0,
+                 build_if_missing=False):
+        if dtype not in ("bfloat16", "float32"):
+            raise ValueError(f"dtype {dtype!r}: bfloat16 or float32")
+        self.config, self.dtype = config, dtype
+        L = self._L = _lib.load_lm(build_if_missing=build_if_missing)
+        self._layers = (_lib.LmLayer * len(config.layers))(*[l.to_c() for l in config.layers])
+        loop = config.loop or {"start": 0, "stop": 0, "times": 1}
+        cfg = _lib.LmConfig(config.vocab, config.width, len(config.layers), self._layers, int(loop["start"]), int(loop["stop"]), int(loop["times"]),
+                            config.norm_eps, max_tokens, max_seqs, max_step_tokens, page_tokens, _lib.LM_F32 if dtype == "float32" else 0)
+        h = C.c_void_p()
+        check(L.zg_lm_create(C.byref(h), C.byref(cfg), device))
+        self.h = h
+        self.n_passes = len(config.passes())
+
+    @classmethod
+    def from_dir(cls, path, dtype="bfloat16", **kw):
+        """config.json + model.safetensors of a checkpoint folder."""
+        from . import weights_io
+
+        m = cls(LMConfig.from_dir(path), dtype=dtype, **kw)
+        m.load_weights(weights_io.load_safetensors_f32(os.path.join(path, "model.safetensors")))
+        return m
+
+    def close(self):
+        if getattr(self, "h", None):
+            self._L.zg_lm_destroy(self.h)
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    # ------------------------------------------------------------------ weights
+    def load_weights(self, weights, strict=True):
+        """weights: dict checkpoint name -> array (fp32 values; matrices [out, in]).  strict: every tensor of the configuration
+        must be there, with its shape, and nothing else."""
+        shapes = self.config.tensor_shapes()
+        for name, a in weights.items():
+            if name not in shapes:
+                if strict:
+                    raise KeyError(f"tensor {name!r} is not part of this configuration")
+                continue
+            if tuple(np.shape(a)) != tuple(shapes[name]):
+                raise ValueError(f"tensor {name!r} has shape {tuple(np.shape(a))}, the configuration needs {tuple(shapes[name])}")
+            a = np.ascontiguousarray(a, dtype=np.float32)
+            check(self._L.zg_lm_load_tensor(self.h, name.encode(), a.ctypes.data, a.size))
+        if strict:
+            missing = self.missing_tensors()
+            if missing:
+                raise KeyError(f"{len(missing)} tensors missing from the checkpoint: {' '.join(missing[:8])}")
+
+    def missing_tensors(self):
+        n, buf = C.c_size_t(), C.create_string_buffer(1 << 16)
+        check(self._L.zg_lm_missing_tensors(self.h, C.byref(n), buf, len(buf)))
+        return buf.value.decode().split() if n.value else []
+
+    def init_random(self, seed=0, std=0.02):
+        check(self._L.zg_lm_init_random(self.h, seed, std))
+
+    # ------------------------------------------------------------------ sequences and steps
+    def open(self):
+        s = C.c_int()
+        check(self._L.zg_lm_seq_open(self.h, C.byref(s)))
+        return s.value
+
+    def close_seq(self, seq):
+        check(self._L.zg_lm_seq_close(self.h, seq))
+
+    def seq_len(self, seq):
+        n = C.c_size_t()
+        check(self._L.zg_lm_seq_len(self.h, seq, C.byref(n)))
+        return n.value
+
+    def free_tokens(self):
+        n = C.c_size_t()
+        check(self._L.zg_lm_free_tokens(self.h, C.byref(n)))
+        return n.value
+
+    def step(self, entries, trace=False):
+        """entries: [(seq, tokens, want)] — the next tokens of every sequence and the places among them whose logits are asked
+        for.  Returns the logits [sum of wants, vocab] in entry order then want order (with trace=True also the residual stream
+        behind every layer pass, [passes, rows, width])."""
+        arr = (_lib.LmEntry * max(1, len(entries)))()
+        keep, n_want, rows = [], 0, 0
+        for i, (seq, tokens, want) in enumerate(entries):
+            t = np.ascontiguousarray(tokens, dtype=np.int32).reshape(-1)
+            w = np.ascontiguousarray(want, dtype=np.int32).reshape(-1)
+            keep += [t, w]
+            arr[i] = _lib.LmEntry(int(seq), t.ctypes.data if t.size else None, t.size, w.ctypes.data if w.size else None, w.size)
+            n_want += w.size
+            rows += t.size
+        logits = np.empty((n_want, self.config.vocab), np.float32)
+        tr = None
+        if trace:
+            tr = np.zeros((self.n_passes, rows, self.config.width), np.float32)
+            check(self._L.zg_lm_set_trace(self.h, tr.ctypes.data, tr.size))
+        try:
+            check(self._L.zg_lm_step(self.h, arr, len(entries), logits.ctypes.data if n_want else None, logits.size))
+        finally:
+            if trace:
+                self._L.zg_lm_set_trace(self.h, None, 0)
+        return (logits, tr) if trace else logits
+
+    def generate(self, prompts, n_new, temp=0.0, seed=0):
+        """Greedy (temp == 0) or sampled continuation of every prompt; returns tokens [len(prompts), n_new]."""
+        prompts = [np.ascontiguousarray(p, dtype=np.int32).reshape(-1) for p in prompts]
+        stride = max(len(p) for p in prompts)
+        mat = np.zeros((len(prompts), stride), np.int32)
+        lens = np.zeros(len(prompts), np.uint64)
+        for b, p in enumerate(prompts):
+            mat[b, : len(p)] = p
+            lens[b] = len(p)
+        out = np.zeros((len(prompts), n_new), np.int32)
+        check(self._L.zg_lm_generate(self.h, mat.ctypes.data, stride, lens.ctypes.data, len(prompts), n_new, float(temp), int(seed), out.ctypes.data,
+                                     out.size))
+        return out
+
+    def last_ms(self):
+        """(device ms of the last step, mean device ms per decode step of the last generate)."""
+        a, b = C.c_float(), C.c_float()
+        check(self._L.zg_lm_last_ms(self.h, C.byref(a), C.byref(b)))
+        return a.value, b.value
+
+    def last_kernel(self):
+        buf = C.create_string_buffer(160)
+        self._L.zg_debug_last_kernel(buf, len(buf))
+        return buf.value.decode()

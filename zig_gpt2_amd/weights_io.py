@@ -63,3 +63,90 @@ def flags_for_checkpoint(weights):
     own precision (src/main.zig:210-269 keeps fp32).  Returns keyword arguments for gpt.GPT."""
     mats = [v for k, v in weights.items() if np.ndim(v) == 2]
     return {"weights_f32": not all(bf16_representable(m) for m in mats)}
+
+
+# ------------------------------------------------------------------------------------------------
+# safetensors checkpoints (the layered models of lm.py): an 8-byte little-endian header length, that many bytes of JSON
+# (tensor name -> dtype, shape, data_offsets relative to the end of the header), then the raw little-endian data.
+# Read with numpy alone; nothing in the file is executed.
+# ------------------------------------------------------------------------------------------------
+_ST_DTYPES = {"F32": ("<f4", 4), "F16": ("<f2", 2), "BF16": ("<u2", 2), "I32": ("<i4", 4), "I64": ("<i8", 8), "F64": ("<f8", 8),
+              "U8": ("u1", 1), "I8": ("i1", 1), "U16": ("<u2", 2), "I16": ("<i2", 2), "U32": ("<u4", 4), "BOOL": ("u1", 1)}
+
+
+def read_safetensors(path):
+    """dict name -> (dtype string of the file, numpy array).  BF16 tensors come back as their uint16 bit patterns (numpy has
+    no bfloat16); everything else in its own type.  The arrays are views of one memory map of the file."""
+    import json
+    import struct
+
+    with open(path, "rb") as f:
+        head = f.read(8)
+        if len(head) != 8:
+            raise ValueError(f"{path}: too short for a safetensors header")
+        (n,) = struct.unpack("<Q", head)
+        size = os.path.getsize(path)
+        if n > size - 8:
+            raise ValueError(f"{path}: header length {n} exceeds the file")
+        meta = json.loads(f.read(n).decode("utf-8"))
+    data = np.memmap(path, dtype=np.uint8, mode="r", offset=8 + n) if size > 8 + n else np.zeros(0, np.uint8)
+    out = {}
+    for name, info in meta.items():
+        if name == "__metadata__":
+            continue
+        if info["dtype"] not in _ST_DTYPES:
+            raise ValueError(f"{path}: tensor {name} has unsupported dtype {info['dtype']}")
+        dt, width = _ST_DTYPES[info["dtype"]]
+        lo, hi = info["data_offsets"]
+        count = int(np.prod(info["shape"], dtype=np.int64)) if info["shape"] else 1
+        if hi - lo != count * width or hi > data.size:
+            raise ValueError(f"{path}: tensor {name}: {hi - lo} bytes on disk, shape {info['shape']} needs {count * width}")
+        out[name] = (info["dtype"], np.frombuffer(data, dtype=dt, count=count, offset=lo).reshape(info["shape"]))
+    return out
+
+
+def bf16_bits_to_f32(bits):
+    """uint16 bf16 bit patterns -> fp32 values (exact)."""
+    return (np.ascontiguousarray(bits, dtype=np.uint16).astype(np.uint32) << np.uint32(16)).view(np.float32)
+
+
+def load_safetensors_f32(path):
+    """dict name -> fp32 array (integer tables stay integer): the form the model classes' load_weights take."""
+    out = {}
+    for name, (dt, a) in read_safetensors(path).items():
+        if dt == "BF16":
+            out[name] = bf16_bits_to_f32(a)
+        elif dt in ("F16", "F64", "F32"):
+            out[name] = np.ascontiguousarray(a, dtype=np.float32)
+        else:
+            out[name] = np.ascontiguousarray(a)
+    return out
+
+
+def write_safetensors(path, tensors, bf16=True):
+    """Write fp32 arrays as BF16 (rounded to nearest even; bf16=False: F32) and integer arrays as I32 — the inverse of
+    load_safetensors_f32 for the layered models' checkpoints."""
+    import json
+    import struct
+
+    from .synth import to_bf16_bits
+
+    meta, blobs, off = {}, [], 0
+    for name, a in tensors.items():
+        a = np.asarray(a)
+        if np.issubdtype(a.dtype, np.integer):
+            dt, raw = "I32", np.ascontiguousarray(a, dtype="<i4").tobytes()
+        elif bf16:
+            dt, raw = "BF16", to_bf16_bits(np.ascontiguousarray(a, dtype=np.float32)).astype("<u2").tobytes()
+        else:
+            dt, raw = "F32", np.ascontiguousarray(a, dtype="<f4").tobytes()
+        meta[name] = {"dtype": dt, "shape": list(a.shape), "data_offsets": [off, off + len(raw)]}
+        blobs.append(raw)
+        off += len(raw)
+    head = json.dumps(meta, separators=(",", ":")).encode("utf-8")
+    head += b" " * (-len(head) % 8)
+    with open(path, "wb") as f:
+        f.write(struct.pack("<Q", len(head)))
+        f.write(head)
+        for b in blobs:
+            f.write(b)
