@@ -123,6 +123,23 @@ def latent_attention(h, w, p, m, eps, positions, cache):
     return o @ w[p + "o"].T, (c_all, kr_all)
 
 
+def attention_weights(h, w, p, m, eps, positions):
+    """The softmax weights [heads, queries, keys] of latent_attention for a whole sequence (tests look at where they peak)."""
+    H, D, R, KR = m["heads"], m["dim"], m["rot_dim"], m["kv_rank"]
+    T = h.shape[0]
+    q = (norm_plain(h @ w[p + "dq"].T, w[p + "dq.norm"], eps) @ w[p + "uq"].T).reshape(T, H, D + R)
+    kv = h @ w[p + "dkv"].T
+    c = norm_plain(kv[:, :KR], w[p + "dkv.norm"], eps)
+    cos, sin = rotary_tables(m["rot"], positions)
+    dims = int(m["rot"]["dims"])
+    kr, qr = rotate_pairs(kv[:, KR:], cos, sin, dims), rotate_pairs(q[:, :, D:], cos, sin, dims)
+    k = (c @ w[p + "uk"].T).reshape(T, H, D)
+    s = (np.einsum("thd,nhd->htn", q[:, :, :D], k) + np.einsum("thr,nr->htn", qr, kr)) * float(m["scale"])
+    s = np.where(np.arange(T)[None, :] <= np.arange(T)[:, None], s, -np.inf)
+    e = np.exp(s - s.max(axis=-1, keepdims=True))
+    return e / e.sum(axis=-1, keepdims=True)
+
+
 # ----------------------------------------------------------------------------------------------- feed-forward
 def dense_ff(h, w, p):
     u = np.maximum(h @ w[p + "up"].T, 0.0)
