@@ -44,6 +44,10 @@ def parse():
     p.add_argument("--no-other-configs", action="store_true", help="skip the secondary block (8 prompts, XL, nano-char)")
     p.add_argument("--cpu-seconds", type=float, default=12.0, help="budget for the CPU baseline sample")
     p.add_argument("--seed", type=int, default=0)
+    p.add_argument("--lm", default="", choices=["", "small", "medium", "large"],
+                   help="instead of the default workload: prompt and decode throughput of a layered model (Tokosun design, random weights) "
+                        "at a size that resembles GPT-2 124M / medium / XL, beside the GPT-2 model of the same width and depth")
+    p.add_argument("--lm-dtype", default="bfloat16", choices=["bfloat16", "float32"])
     p.add_argument("--dry-run", action="store_true",
                    help="CPU rehearsal of the launch path (gloo, no GPU, no kernels): rendezvous, prompt sharding, "
                         "weight-arena broadcast, barriers and the max-reduce; prints a line with dry_run=true")
@@ -415,6 +419,131 @@ def groups_table(seed, n_prompts=8, group_counts=(1, 2, 4, 8)):
     return [best[g] for g in group_counts]
 
 
+# ------------------------------------------------------------------------------------------------
+# --lm: the layered-model tier (zig_gpt2_amd/lm.py) at sizes that resemble real models, beside GPT-2 of equal width and depth
+# ------------------------------------------------------------------------------------------------
+LM_SIZES = {"small": ("124M", 768, 12), "medium": ("medium", 1024, 24), "large": ("xl", 1600, 48)}
+
+
+def lm_bench_config(width, n_layers, vocab):
+    """A Tokosun-design stack of `n_layers` layers in the repeating order recurrence + dense, attention + experts, attention +
+    experts, recurrence + experts, with head sizes of 64 to 128 channels, a dense feed-forward of 4 x width and 8 experts of
+    width `width` of which 2 are chosen (24 W^2 stored, 6 W^2 active per layer)."""
+    from zig_gpt2_amd import lm
+
+    hd = 128 if width % 128 == 0 else 64
+    rec = dict(mixer="hgrn2", heads=width // hd, dim=hd, vdim=hd)
+    att = dict(mixer="latent_attention", heads=width // 64, dim=64, vdim=64, rot_dim=32, kv_rank=256, q_rank=384, scale=(64 + 32) ** -0.5,
+               rot_dims=32, rot_base=10000.0, rot_scaling={"factor": 4.0, "original": 2048, "fast": 32.0, "slow": 1.0})
+    dense = dict(ff="dense", ff_width=4 * width)
+    moe = dict(ff="moe", ff_width=width, experts=8, top=2)
+    order = [dict(rec, **dense), dict(att, **moe), dict(att, **moe), dict(rec, **moe)]
+    return lm.LMConfig(vocab=vocab, width=width, layers=[lm.LayerSpec(**order[i % 4]) for i in range(n_layers)], norm_eps=1e-6)
+
+
+def lm_weight_bytes(cfg):
+    """(stored, read per decoded token) bytes of the bf16 matrices: every expert is stored, `top` of them are read."""
+    stored = active = 0
+    for name, shape in cfg.tensor_shapes().items():
+        if len(shape) != 2 or name == "embed":
+            continue
+        b = 2 * shape[0] * shape[1]
+        stored += b
+        if ".mlp.e" in name:
+            lay = cfg.layers[int(name[1:name.index(".")])]
+            b = b * lay.top / lay.experts
+        active += b
+    return int(stored), int(active)
+
+
+def lm_bench(a):
+    import torch
+
+    from zig_gpt2_amd import _lib, gpt, lm, synth
+
+    assert torch.cuda.is_available(), "bench.py needs an MI355X"
+    gname, width, n_layers = LM_SIZES[a.lm]
+    gcfg = synth.CONFIGS.get(gname) or synth.GPTConfig(50257, 1024, n_layers, width // 64, width)
+    ctx = a.ctx or 1024
+    cfg = lm_bench_config(width, n_layers, gcfg.vocab_size)
+    out = {"metric": "lm_decode_tokens_per_s", "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "higher_is_better": True,
+           "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if a.lm_dtype == "bfloat16" else "fp32", "data": "synthetic (random weights, filled on the GPU)",
+           "config": {"model": f"Tokosun design, width {width}, {n_layers} layers (recurrence+dense, attention+experts x2, recurrence+experts), vocab {gcfg.vocab_size}",
+                      "global_batch": 1, "seq_len": ctx, "parallelism": "single GPU"}}
+    m = lm.LayeredLM(cfg, dtype=a.lm_dtype, max_tokens=8 * ctx + 64, max_seqs=8, max_step_tokens=8 * ctx)
+    m.init_random(seed=a.seed + 1, std=0.02)
+    stored, active = lm_weight_bytes(cfg)
+    rng = np.random.default_rng(a.seed)
+
+    def prompt_pass(n_prompts, n):
+        toks = [rng.integers(0, cfg.vocab, n).astype(np.int32) for _ in range(n_prompts)]
+        best_wall = best_dev = 1e30
+        for it in range(a.warmup + a.steps):
+            seqs = [m.open() for _ in toks]
+            t0 = time.perf_counter()
+            m.step([(s, t, [n - 1]) for s, t in zip(seqs, toks)])
+            wall = (time.perf_counter() - t0) * 1e3
+            for s in seqs:
+                m.close_seq(s)
+            if it >= a.warmup:
+                best_wall, best_dev = min(best_wall, wall), min(best_dev, m.last_ms()[0])
+        return {"prompts": n_prompts, "prompt_tokens": n, "ms": round(best_wall, 3), "device_ms": round(best_dev, 3),
+                "prompt_tokens_per_s": round(n_prompts * n / best_wall * 1e3, 1)}
+
+    def decode(n_prompts):
+        prompts = [rng.integers(0, cfg.vocab, 1).astype(np.int32) for _ in range(n_prompts)]
+        best = None
+        for it in range(a.warmup + a.steps):
+            t0 = time.perf_counter()
+            m.generate(prompts, ctx - 1)
+            wall = time.perf_counter() - t0
+            r = {"prompts": n_prompts, "decode_steps": ctx - 1, "tokens_per_s": round(n_prompts * (ctx - 1) / wall, 1),
+                 "device_us_per_step": round(m.last_ms()[1] * 1e3, 1), "wall_us_per_step": round(wall / (ctx - 1) * 1e6, 1)}
+            if it >= a.warmup and (best is None or r["tokens_per_s"] > best["tokens_per_s"]):
+                best = r
+        best["weight_bytes_per_step"] = active if n_prompts == 1 else None
+        best["frac_of_8TBps_weights_only"] = round(active / (best["device_us_per_step"] * 1e-6) / 1e9 / HBM_PEAK_GBS, 4) if n_prompts == 1 else None
+        return best
+
+    lm_res = {"weights_bytes_stored": stored, "weights_bytes_read_per_token": active,
+              "prefill": [prompt_pass(1, ctx - 1), prompt_pass(8, ctx - 1), prompt_pass(1, 128)], "decode": [decode(1), decode(8)]}
+    m.close()
+
+    # GPT-2 of the same width and depth through its own tier (captured decode graphs, whole-prompt pass)
+    lib = _lib.load()
+    _lib.check(lib.zg_init(0))
+    g_res = {"config": f"GPT-2 width {gcfg.n_embed}, {gcfg.n_layer} layers, {gcfg.n_heads} heads", "prefill": [], "decode": []}
+    w = device_weights(gcfg, a.seed)
+    for ppg in (1, 8):
+        model = gpt.GPT(gcfg, batch=ppg)
+        try:
+            model.load_weights(w)
+            prompts = [synth.rand_tokens(2000 + b, 1, gcfg.vocab_size) for b in range(ppg)]
+            best = 1e30
+            for it in range(a.warmup + a.steps):
+                t0 = time.perf_counter()
+                model.generate(prompts, ctx)
+                if it >= a.warmup:
+                    best = min(best, time.perf_counter() - t0)
+            g_res["decode"].append({"prompts": ppg, "decode_steps": ctx, "tokens_per_s": round(ppg * (ctx - 1) / best, 1),
+                                    "wall_us_per_step": round(best / ctx * 1e6, 1)})
+            for n in ((ctx - 1, 128) if ppg == 1 else (ctx - 1,)):
+                ptoks = np.stack([synth.rand_tokens(3000 + b, n, gcfg.vocab_size) for b in range(ppg)])
+                best = 1e30
+                for it in range(a.warmup + a.steps):
+                    t0 = time.perf_counter()
+                    model.prefill(ptoks, compute_logits=True, want_logits=False)
+                    lib.zg_synchronize()
+                    if it >= a.warmup:
+                        best = min(best, (time.perf_counter() - t0) * 1e3)
+                g_res["prefill"].append({"prompts": ppg, "prompt_tokens": n, "ms": round(best, 3), "prompt_tokens_per_s": round(ppg * n / best * 1e3, 1)})
+        finally:
+            model.close()
+    d1 = lm_res["decode"][0]
+    out.update(value=d1["tokens_per_s"], ms_per_step=round(d1["wall_us_per_step"] / 1e3, 4), tokosun=lm_res, gpt2_equal_size=g_res)
+    print(json.dumps(out))
+
+
 def prefill_flops(cfg, prompts, n, ms, planes=3):
     """Matrix-core work of one whole-prompt pass: the useful Linear FLOPs (2 M K N each), and what the MFMAs execute — `planes`
     bf16 plane products per Linear (exact split of the fp32 activations), six per attention product (both operands split),
@@ -440,6 +569,8 @@ def main():
         sys.exit(2)
     if a.dry_run:
         return dry_run(a, rank, world)
+    if a.lm:
+        return lm_bench(a)
     # The two measurements that run as CHILD processes are taken first, while this process holds no GPU queue: both are sensitive
     # to who else has queues on the device (the co-running groups: DESIGN §3.3; the op tier polls a completion word behind every
     # call — under a parent with a dozen idle queues it has read 600 tok/s where it reads 770-850 alone).

@@ -368,7 +368,10 @@ typedef struct {
     int ff_width;                 /* hidden width of the dense feed-forward, or of ONE expert */
     int experts, top;
 } zg_lm_layer;
-enum { ZG_LM_F32 = 1 << 0 /* true 32-bit products everywhere */ };
+enum {
+    ZG_LM_F32 = 1 << 0,     /* true 32-bit products everywhere */
+    ZG_LM_NO_GRAPH = 1 << 1 /* launch the kernels of a decode step one by one instead of replaying the hipGraph captured for its batch size */
+};
 typedef struct {
     size_t vocab, width, n_layers;
     const zg_lm_layer* layers;

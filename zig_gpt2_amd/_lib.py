@@ -66,7 +66,7 @@ class LmEntry(C.Structure):
 
 LM_MIX_HGRN2, LM_MIX_LATENT_ATTENTION = 1, 2
 LM_FF_NONE, LM_FF_DENSE, LM_FF_MOE = 0, 1, 2
-LM_F32 = 1
+LM_F32, LM_NO_GRAPH = 1, 2
 
 # the layered-model tier (present in both libraries)
 LM_SIGNATURES = {

@@ -145,7 +145,11 @@ struct zg_lm {
     // scratch
     float *x = nullptr, *h = nullptr, *y = nullptr, *proj = nullptr, *cq = nullptr, *q = nullptr, *qa = nullptr, *ctx = nullptr, *o = nullptr, *u = nullptr;
     float *gu_buf = nullptr, *hb = nullptr, *ye = nullptr, *wt = nullptr, *last_h = nullptr, *hn = nullptr, *logits = nullptr;
-    float *row_max = nullptr, *samp_ws = nullptr, *samp_u = nullptr;
+    float *row_max = nullptr, *samp_ws = nullptr, *samp_u = nullptr, *amax_val = nullptr;
+    int* amax_idx = nullptr;
+    float *attn_ws = nullptr, *scan_ws = nullptr;
+    size_t scan_ws_floats = 0;
+    size_t attn_ws_floats = 0;
     int *pick = nullptr, *grp_off = nullptr, *sorted = nullptr, *inv = nullptr, *tok_out = nullptr, *flag = nullptr;
     int* meta = nullptr;    // device: ids | pos | slot | prev | last-entry | want rows | entry start | entry len | entry slot
     int* h_meta = nullptr;  // pinned twin
@@ -155,6 +159,8 @@ struct zg_lm {
     float* trace = nullptr;
     size_t trace_floats = 0;
     float last_step_ms = 0.0f, last_decode_ms = 0.0f;
+    bool use_graph = true;
+    hipGraphExec_t decode_graph[kGemvMaxRows + 1] = {};  // by rows of the step (one per entry)
 };
 
 namespace {
@@ -190,7 +196,7 @@ void layout(zg_lm* g, Bump& b) {
     g->head = b.take<bf16_t>(V * W);
     mat("head", g->head, 0, V, W);
     vec("final.norm", g->final_norm, W, INIT_OFFSET);
-    size_t max_proj = 1, max_qr = 1, max_q = 1, max_qa = 1, max_ctx = 1, max_o = 1, max_ff = 1, max_assign = 1, max_gu = 1, max_hb = 1, max_e = 1;
+    size_t max_proj = 1, max_qr = 1, max_q = 1, max_qa = 1, max_ctx = 1, max_o = 1, max_ff = 1, max_assign = 1, max_gu = 1, max_hb = 1, max_e = 1, max_att_part = 0, max_scan = 0;
     for (size_t i = 0; i < g->layers.size(); ++i) {
         LayerW& L = g->layers[i];
         const zg_lm_layer& d = L.d;
@@ -211,6 +217,7 @@ void layout(zg_lm* g, Bump& b) {
             L.o = b.take<bf16_t>(W * HV);
             mat(p + "mix.o", L.o, 0, W, HV);
             max_proj = std::max(max_proj, 2 * HD + HV);
+            max_scan = std::max(max_scan, H * D * Vd + H * D);
             max_o = std::max(max_o, HV);
         } else {
             const size_t R = d.rot_dim, KR = d.kv_rank, QR = d.q_rank, HV = H * Vd;
@@ -233,6 +240,7 @@ void layout(zg_lm* g, Bump& b) {
             max_q = std::max(max_q, H * (D + R));
             max_qa = std::max(max_qa, H * (KR + R));
             max_ctx = std::max(max_ctx, H * KR);
+            max_att_part = std::max(max_att_part, H * (KR + 2));
             max_o = std::max(max_o, HV);
         }
         if (d.ff != ZG_LM_FF_NONE) {
@@ -301,6 +309,10 @@ void layout(zg_lm* g, Bump& b) {
     g->sorted = b.take<int>(MS * max_assign);
     g->inv = b.take<int>(MS * max_assign);
     g->grp_off = b.take<int>(max_e + 1);
+    g->scan_ws_floats = (MS / 64 + 1 + NS) * max_scan;
+    g->scan_ws = b.take<float>(std::max<size_t>(1, g->scan_ws_floats));
+    g->attn_ws_floats = (size_t)kGemvMaxRows * kAttnSplits * max_att_part;
+    g->attn_ws = b.take<float>(std::max<size_t>(1, g->attn_ws_floats));
     g->last_h = b.take<float>((size_t)g->n_passes * NS * W);
     g->hn = b.take<float>((size_t)g->logit_rows * W);
     g->logits = b.take<float>((size_t)g->logit_rows * V);
@@ -308,6 +320,8 @@ void layout(zg_lm* g, Bump& b) {
     g->samp_ws = b.take<float>(sample_workspace_floats(g->logit_rows));
     g->samp_u = b.take<float>(g->logit_rows);
     g->tok_out = b.take<int>(g->logit_rows);
+    g->amax_val = b.take<float>((size_t)g->logit_rows * kArgmaxParts);
+    g->amax_idx = b.take<int>((size_t)g->logit_rows * kArgmaxParts);
     g->flag = b.take<int>(16);
     g->meta = b.take<int>(meta_ints(g));
 }
@@ -358,42 +372,17 @@ int check_layer(const zg_lm_layer& d, size_t i) {
     return ZG_OK;
 }
 
-// ------------------------------------------------------------------------------------------------ one portion of rows
-int run_portion(zg_lm* g, const std::vector<Piece>& pieces, float* logits_out, const Sampler* sampler) {
+// The kernels of one portion, from the embedding to the commit of the token-shift rows: launches only, every per-step value
+// (tokens, positions, slots, page tables) is read from device memory — so for a given number of rows and entries the sequence
+// is the same every step and can be replayed from a captured graph (decode steps: one row per entry).
+int enqueue_layers(zg_lm* g, int M, int n_ent, bool capturing) {
     hipStream_t s = g->stream;
     const int W = g->W, MS = g->MS, NS = g->NS;
-    int M = 0;
-    for (const Piece& pc : pieces) M += pc.n;
-    if (M == 0) return ZG_OK;
-    const int n_ent = (int)pieces.size();
-    int *ids = g->h_meta, *pos = ids + MS, *slot = pos + MS, *prev = slot + MS, *lastent = prev + MS, *want_rows = lastent + MS;
-    int *ent_start = want_rows + MS, *ent_len = ent_start + NS, *ent_slot = ent_len + NS;
-    std::vector<std::pair<int, size_t>> wants;  // (row of the portion, output row)
-    int r = 0;
-    for (int e = 0; e < n_ent; ++e) {
-        const Piece& pc = pieces[e];
-        ent_start[e] = r;
-        ent_len[e] = pc.n;
-        ent_slot[e] = pc.slot;
-        for (int t = 0; t < pc.n; ++t, ++r) {
-            ids[r] = pc.tok[t];
-            pos[r] = pc.pos0 + t;
-            slot[r] = pc.slot;
-            prev[r] = t > 0 ? r - 1 : -1;
-            lastent[r] = t == pc.n - 1 ? e : -1;
-        }
-        for (auto& w : pc.wants) wants.push_back({ent_start[e] + w.first, w.second});
-        const Slot& sl = g->slots[pc.slot];
-        ZG_HIP(hipMemcpyAsync(g->page_table + (size_t)pc.slot * g->max_pages, sl.pages.data(), sl.pages.size() * sizeof(int), hipMemcpyHostToDevice, s));
-    }
-    ZG_HIP(hipMemcpyAsync(g->meta, g->h_meta, meta_ints(g) * sizeof(int), hipMemcpyHostToDevice, s));
     const int *d_ids = g->meta, *d_pos = d_ids + MS, *d_slot = d_pos + MS, *d_prev = d_slot + MS, *d_last = d_prev + MS, *d_want = d_last + MS;
     const int *d_estart = d_want + MS, *d_elen = d_estart + NS, *d_eslot = d_elen + NS;
     const bool f32 = g->f32;
     const float eps = g->cfg.norm_eps;
     const bool few = M <= kGemvMaxRows;
-
-    ZG_HIP(hipEventRecord(g->ev0, s));
     ZG_TRY(launch_embed(g->embed, d_ids, g->x, M, W, g->V, g->flag, s));
     for (int p = 0; p < g->n_passes; ++p) {
         const Pass& ps = g->passes[p];
@@ -409,7 +398,8 @@ int run_portion(zg_lm* g, const std::vector<Piece>& pieces, float* logits_out, c
             lin.A = g->h; lin.lda = W; lin.B = L.qfv; lin.ldb = W; lin.C = g->proj; lin.ldc = NP; lin.M = M; lin.N = NP; lin.K = W;
             ZG_TRY(launch_linear(lin, f32, s));
             ZG_TRY(launch_hgrn2_gates(g->proj, NP, M, HD, L.fb, L.lower, s));
-            ZG_TRY(launch_hgrn2_scan(g->proj, NP, g->o, HV, g->hgrn_state + ps.hgrn_off, g->hgrn_floats, d_estart, d_elen, d_eslot, n_ent, H, D, Vd, s));
+            ZG_TRY(launch_hgrn2_scan(g->proj, NP, g->o, HV, g->hgrn_state + ps.hgrn_off, g->hgrn_floats, d_estart, d_elen, d_eslot, n_ent, M, H, D, Vd,
+                                     g->scan_ws, g->scan_ws_floats, s));
             ZG_TRY(launch_norm_plain(g->o, HV, H, Vd, M, L.hnorm, eps, s));
             lin = Linear();
             lin.A = g->o; lin.lda = HV; lin.B = L.o; lin.ldb = HV; lin.C = g->y; lin.ldc = W; lin.M = M; lin.N = W; lin.K = HV;
@@ -430,7 +420,13 @@ int run_portion(zg_lm* g, const std::vector<Piece>& pieces, float* logits_out, c
             lin.C = g->qa; lin.ldc = H * (KR + R); lin.c_zoff = KR + R; lin.M = M; lin.N = KR; lin.K = D; lin.nz = H;
             ZG_TRY(launch_linear(lin, f32, s));
             ZG_TRY(launch_q_rotary(g->q, H * (D + R), g->qa, H * (KR + R), M, H, D, R, KR, rot, d_pos, s));
-            ZG_TRY(launch_latent_attention(g->qa, g->ctx, M, H, KR, R, d.scale, d_pos, d_slot, g->page_table, g->max_pages, g->P, ps.cache, nullptr, 0, s));
+            bool tiled = false;
+            if (!f32 && !few)
+                ZG_TRY(launch_latent_attention_tiles(g->qa, g->ctx, M, H, KR, R, d.scale, d_estart, d_elen, d_eslot, n_ent, d_pos, g->page_table,
+                                                     g->max_pages, g->P, ps.cache, s, &tiled));
+            if (!tiled)
+                ZG_TRY(launch_latent_attention(g->qa, g->ctx, M, H, KR, R, d.scale, d_pos, d_slot, g->page_table, g->max_pages, g->P, ps.cache,
+                                               g->attn_ws, g->attn_ws_floats, s));
             lin = Linear();  // values of the weighted latent, head by head
             lin.A = g->ctx; lin.lda = H * KR; lin.a_zoff = KR; lin.B = L.uv; lin.ldb = KR; lin.b_zoff = (long long)Vd * KR;
             lin.C = g->o; lin.ldc = HV; lin.c_zoff = Vd; lin.M = M; lin.N = Vd; lin.K = KR; lin.nz = H;
@@ -470,13 +466,71 @@ int run_portion(zg_lm* g, const std::vector<Piece>& pieces, float* logits_out, c
             ZG_TRY(launch_linear(dn, f32, s));
             ZG_TRY(launch_moe_combine(g->x, g->ye, few ? nullptr : g->inv, g->wt, top, L.norm2b, eps, M, W, s));
         }
-        if (g->trace && (size_t)(p + 1) * M * W <= g->trace_floats) {
+        if (g->trace && !capturing && (size_t)(p + 1) * M * W <= g->trace_floats) {
             ZG_HIP(hipMemcpyAsync(g->trace + (size_t)p * M * W, g->x, (size_t)M * W * sizeof(float), hipMemcpyDeviceToHost, s));
             ZG_HIP(hipStreamSynchronize(s));
         }
     }
     // the rows the last tokens of the entries left for the token shift of their successors
     ZG_TRY(launch_commit_rows(g->shift_state, (size_t)g->n_passes * W, g->last_h, W, d_eslot, n_ent, W, g->n_passes, W, (size_t)NS * W, s));
+
+    return ZG_OK;
+}
+
+// ------------------------------------------------------------------------------------------------ one portion of rows
+int run_portion(zg_lm* g, const std::vector<Piece>& pieces, float* logits_out, const Sampler* sampler) {
+    hipStream_t s = g->stream;
+    const int W = g->W, MS = g->MS, NS = g->NS;
+    int M = 0;
+    for (const Piece& pc : pieces) M += pc.n;
+    if (M == 0) return ZG_OK;
+    const int n_ent = (int)pieces.size();
+    int *ids = g->h_meta, *pos = ids + MS, *slot = pos + MS, *prev = slot + MS, *lastent = prev + MS, *want_rows = lastent + MS;
+    int *ent_start = want_rows + MS, *ent_len = ent_start + NS, *ent_slot = ent_len + NS;
+    std::vector<std::pair<int, size_t>> wants;  // (row of the portion, output row)
+    int r = 0;
+    for (int e = 0; e < n_ent; ++e) {
+        const Piece& pc = pieces[e];
+        ent_start[e] = r;
+        ent_len[e] = pc.n;
+        ent_slot[e] = pc.slot;
+        for (int t = 0; t < pc.n; ++t, ++r) {
+            ids[r] = pc.tok[t];
+            pos[r] = pc.pos0 + t;
+            slot[r] = pc.slot;
+            prev[r] = t > 0 ? r - 1 : -1;
+            lastent[r] = t == pc.n - 1 ? e : -1;
+        }
+        for (auto& w : pc.wants) wants.push_back({ent_start[e] + w.first, w.second});
+        const Slot& sl = g->slots[pc.slot];
+        ZG_HIP(hipMemcpyAsync(g->page_table + (size_t)pc.slot * g->max_pages, sl.pages.data(), sl.pages.size() * sizeof(int), hipMemcpyHostToDevice, s));
+    }
+    ZG_HIP(hipMemcpyAsync(g->meta, g->h_meta, meta_ints(g) * sizeof(int), hipMemcpyHostToDevice, s));
+    const int* d_want = g->meta + 5 * (size_t)MS;
+    const bool f32 = g->f32;
+    const float eps = g->cfg.norm_eps;
+
+    ZG_HIP(hipEventRecord(g->ev0, s));
+    bool single = M <= kGemvMaxRows && !g->trace && g->use_graph;
+    for (const Piece& pc : pieces) single = single && pc.n == 1;
+    if (single) {  // a decode step: replay the captured sequence of this batch size
+        if (!g->decode_graph[M]) {
+            hipGraph_t graph = nullptr;
+            ZG_HIP(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal));
+            const int st = enqueue_layers(g, M, n_ent, true);
+            const hipError_t ce = hipStreamEndCapture(s, &graph);
+            if (st != ZG_OK) {
+                if (graph) (void)hipGraphDestroy(graph);
+                return st;
+            }
+            ZG_HIP(ce);
+            ZG_HIP(hipGraphInstantiate(&g->decode_graph[M], graph, nullptr, nullptr, 0));
+            ZG_HIP(hipGraphDestroy(graph));
+        }
+        ZG_HIP(hipGraphLaunch(g->decode_graph[M], s));
+    } else {
+        ZG_TRY(enqueue_layers(g, M, n_ent, false));
+    }
 
     // logits of the rows that were asked for, logit_rows at a time
     size_t w0 = 0;
@@ -492,7 +546,7 @@ int run_portion(zg_lm* g, const std::vector<Piece>& pieces, float* logits_out, c
             lin.A = g->hn; lin.lda = W; lin.B = g->head; lin.ldb = W; lin.C = g->logits; lin.ldc = g->V; lin.M = nw; lin.N = g->V; lin.K = W;
             ZG_TRY(launch_linear(lin, f32, s));
             if (sampler) {
-                ZG_TRY(launch_row_argmax(g->logits, nw, g->V, g->row_max, g->tok_out, s));
+                ZG_TRY(launch_row_argmax(g->logits, nw, g->V, g->row_max, g->tok_out, g->amax_val, g->amax_idx, s));
                 if (sampler->temp > 0.0f) {
                     for (int j = 0; j < nw; ++j) {  // the uniform of (seed, length of the sequence with the token to be drawn, output row)
                         const int row = wants[w0 + j].first;
@@ -616,6 +670,7 @@ int zg_lm_create(zg_lm** out, const zg_lm_config* config, int device) {
     g->cfg = *config;
     g->device = device;
     g->f32 = (config->flags & ZG_LM_F32) != 0;
+    g->use_graph = (config->flags & ZG_LM_NO_GRAPH) == 0;
     g->W = (int)config->width;
     g->V = (int)config->vocab;
     g->MS = (int)(config->max_step_tokens ? config->max_step_tokens : 2048);
@@ -708,6 +763,8 @@ int zg_lm_destroy(zg_lm* g) {
     if (!g) return ZG_OK;
     (void)hipSetDevice(g->device);
     if (g->stream) (void)hipStreamSynchronize(g->stream);
+    for (hipGraphExec_t e : g->decode_graph)
+        if (e) (void)hipGraphExecDestroy(e);
     if (g->ev0) (void)hipEventDestroy(g->ev0);
     if (g->ev1) (void)hipEventDestroy(g->ev1);
     if (g->stream) (void)hipStreamDestroy(g->stream);

@@ -72,8 +72,10 @@ int launch_norm_plain(float* v, int ld, int rows_per_m, int width, int M, const 
 int launch_hgrn2_gates(float* proj, int ld, int M, int HD, const float* bias, const float* low, hipStream_t s);
 // Per entry e (rows ent_start[e] .. + ent_len[e]) and head: S <- diag(f_t) S + (1 - f_t) v_t^T, o_t = S^T q_t, token by token,
 // S = state[ent_slot[e]] ([H][D][V] fp32) read at the start and written back at the end.  out rows [H V], row stride ldo.
+// M: rows of the step.  ws (may be null): workspace for the chunk-parallel form of long steps, (M / 64 + n_entries) * (H D V + H D) floats.
 int launch_hgrn2_scan(const float* proj, int ld, float* out, int ldo, float* state, size_t slot_stride, const int* ent_start,
-                      const int* ent_len, const int* ent_slot, int n_entries, int H, int D, int V, hipStream_t s);
+                      const int* ent_len, const int* ent_slot, int n_entries, int M, int H, int D, int V, float* ws, size_t ws_floats,
+                      hipStream_t s);
 
 // ------------------------------------------------------------------------------------------------ latent attention
 // Rotary table of one layer: freq[i] for the rot_dims / 2 pairs (YaRN blend applied on the host) and the amplitude factor.
@@ -90,9 +92,17 @@ int launch_latent_prep(const float* proj, int ld, int M, int q_rank, int KR, int
 // qa[m][h][KR ..] = rotary(q[m][h][D ..]) — the rotated query part moved behind the absorbed part (which a batched Linear wrote).
 int launch_q_rotary(const float* q, int ldq, float* qa, int ldqa, int M, int H, int D, int R, int KR, Rotary rot, const int* row_pos, hipStream_t s);
 // ctx[m][h][:KR] = sum_j softmax_j( scale * qa[m][h] . cacherow(j) ) latent(j) over the keys j <= row_pos[m] of the row's sequence.
-// ws: fp32 workspace for the partials of split key ranges (decode), ws_floats its size.
+// ws: fp32 workspace for the partials of split key ranges (steps of at most kGemvMaxRows rows: M * H * kAttnSplits * (KR + 2)
+// floats; without it whole key rows per workgroup).
+constexpr int kAttnSplits = 16;
 int launch_latent_attention(const float* qa, float* ctx, int M, int H, int KR, int R, float scale, const int* row_pos, const int* row_slot,
                             const int* page_table, int max_pages, int page_tokens, const float* cache, float* ws, size_t ws_floats, hipStream_t s);
+
+// The same for prompt portions on the matrix cores (bf16 operands, fp32 scores / softmax / accumulation): 32 queries of one entry
+// and four heads per workgroup.  *taken = false when the latent is larger than the kernel's tiles hold (nothing launched).
+int launch_latent_attention_tiles(const float* qa, float* ctx, int M, int H, int KR, int R, float scale, const int* ent_start, const int* ent_len,
+                                  const int* ent_slot, int n_entries, const int* row_pos, const int* page_table, int max_pages, int page_tokens,
+                                  const float* cache, hipStream_t s, bool* taken);
 
 // ------------------------------------------------------------------------------------------------ mixture of experts
 // Per row: z = router . g (fp32), s = softmax(z), the `top` experts by s + correction (lowest index wins a tie), weights s.
@@ -107,8 +117,10 @@ int launch_moe_combine(float* x, const float* yexp, const int* inv, const float*
                        hipStream_t s);
 
 // ------------------------------------------------------------------------------------------------ sampling support
-// Per row: the maximum of its logits and the index of the first element that reaches it.
-int launch_row_argmax(const float* logits, int rows, int n, float* max_out, int* idx_out, hipStream_t s);
+// Per row: the maximum of its logits and the index of the first element that reaches it.  part_val / part_idx: workspace of
+// rows * kArgmaxParts elements each (the row is scanned in slices by that many workgroups, a second launch combines them).
+constexpr int kArgmaxParts = 64;
+int launch_row_argmax(const float* logits, int rows, int n, float* max_out, int* idx_out, float* part_val, int* part_idx, hipStream_t s);
 
 }  // namespace lm
 }  // namespace zg

@@ -3,6 +3,8 @@
 // Everything here is fp32 in both precision modes: norms, gates, the recurrent state, positions, angles, scores and weights.
 #include <math.h>
 
+#include <algorithm>
+
 #include "lm_kernels.h"
 
 namespace zg {
@@ -123,62 +125,141 @@ __global__ __launch_bounds__(256) void hgrn2_gates_kernel(float* proj, int ld, i
     row[HD + i] = l + (1.0f - l) * sigmoid_f(row[HD + i] + bias[i]);
 }
 
-// A column j of a head's state S[D][V] is held by G consecutive lanes, 16 rows each (D <= 16 G); the token loop is serial, the
-// next token's gates are fetched while the current one is applied.
+// A column j of a head's state S[D][V] is held by G consecutive lanes, 16 rows each (D <= 16 G).  The token loop is serial; the
+// gates and values of the next SB tokens are staged in the LDS (rows beyond D padded with q = 0, f = 1: they stay zero).
+//
+// Long entries are cut into chunks of kScanChunk tokens that run side by side (the recurrence is linear in S):
+//   phase A   every chunk from a zero state: its end state B_c and the product A_c of its gates per row
+//   phase B   S_start(c + 1) = A_c * S_start(c) + B_c down the chunks of an entry (elementwise; S_start overwrites B in place)
+//   phase C   every chunk again from its true start state, now writing the outputs
+// Short steps (decoding, small portions) run the same kernel once per entry, from the slot's state and back into it.
 constexpr int kScanRows = 16;
+constexpr int kScanChunk = 64;
+enum { SCAN_DIRECT = 0, SCAN_A = 1, SCAN_C = 2 };
+
+// which (entry, chunk) a workgroup of the chunked phases works on; false: none
+__device__ __forceinline__ bool scan_find_chunk(int id, const int* ent_len, int n_entries, int& e, int& c) {
+    for (e = 0; e < n_entries; ++e) {
+        const int nc = (ent_len[e] + kScanChunk - 1) / kScanChunk;
+        if (id < nc) {
+            c = id;
+            return true;
+        }
+        id -= nc;
+    }
+    return false;
+}
+
 template <int G>
 __global__ __launch_bounds__(256) void hgrn2_scan_kernel(const float* proj, int ld, float* out, int ldo, float* state, size_t slot_stride,
-                                                         const int* ent_start, const int* ent_len, const int* ent_slot, int H, int D, int V) {
-    const int e = blockIdx.x, h = blockIdx.y;
+                                                         const int* ent_start, const int* ent_len, const int* ent_slot, int n_entries, int H, int D,
+                                                         int V, int mode, int SB, float* wsB, float* wsA) {
+    extern __shared__ __attribute__((aligned(16))) float s_scan[];
+    constexpr int Dp = G * kScanRows;
     const int cols = blockDim.x / G;
-    const int j = blockIdx.z * cols + threadIdx.x / G, g = threadIdx.x % G;
+    float* sq = s_scan;             // [SB][Dp]
+    float* sf = sq + SB * Dp;       // [SB][Dp]
+    float* sv = sf + SB * Dp;       // [SB][cols]
+    const int h = blockIdx.y;
+    const int jl = threadIdx.x / G, g = threadIdx.x % G, j0 = blockIdx.z * cols, j = j0 + jl;
     const bool col_ok = j < V;
-    const int HD = H * D, T = ent_len[e], m0 = ent_start[e];
-    float* S_mem = state + (size_t)ent_slot[e] * slot_stride + (size_t)h * D * V;
-    float S[kScanRows];
-    bool ok[kScanRows];
+    const int HD = H * D;
+    int e, c = 0, t_lo, t_hi;
+    if (mode == SCAN_DIRECT) {
+        e = blockIdx.x;
+        t_lo = 0;
+        t_hi = ent_len[e];
+    } else {
+        if (!scan_find_chunk(blockIdx.x, ent_len, n_entries, e, c)) return;
+        t_lo = c * kScanChunk;
+        t_hi = min(ent_len[e], t_lo + kScanChunk);
+    }
+    const int m0 = ent_start[e];
+    const size_t head_floats = (size_t)D * V;
+    float* S_slot = state + (size_t)ent_slot[e] * slot_stride + (size_t)h * head_floats;
+    float* S_ws = wsB ? wsB + ((size_t)blockIdx.x * H + h) * head_floats : nullptr;
+    const float* S_in = mode == SCAN_DIRECT ? S_slot : mode == SCAN_C ? S_ws : nullptr;
+    float S[kScanRows], A[kScanRows];
 #pragma unroll
     for (int r = 0; r < kScanRows; ++r) {
         const int i = g * kScanRows + r;
-        ok[r] = col_ok && i < D;
-        S[r] = ok[r] ? S_mem[(size_t)i * V + j] : 0.0f;
+        S[r] = (S_in && col_ok && i < D) ? S_in[(size_t)i * V + j] : 0.0f;
+        A[r] = 1.0f;
     }
-    const int qoff = h * D + g * kScanRows, foff = HD + qoff, voff = 2 * HD + h * V + j;
-    float q[kScanRows], f[kScanRows], v = 0.0f;
-    auto fetch = [&](int t, float* qd, float* fd, float& vd) {
-        const float* row = proj + (size_t)(m0 + t) * ld;
-#pragma unroll
-        for (int r = 0; r < kScanRows; ++r) {
-            qd[r] = ok[r] ? row[qoff + r] : 0.0f;
-            fd[r] = ok[r] ? row[foff + r] : 1.0f;
+    for (int tb = t_lo; tb < t_hi; tb += SB) {
+        const int nb = min(SB, t_hi - tb);
+        __syncthreads();  // the previous block has been consumed
+        for (int idx = threadIdx.x; idx < nb * Dp; idx += blockDim.x) {
+            const int tt = idx / Dp, i = idx % Dp;
+            const float* row = proj + (size_t)(m0 + tb + tt) * ld;
+            sq[idx] = i < D ? row[h * D + i] : 0.0f;
+            sf[idx] = i < D ? row[HD + h * D + i] : 1.0f;
         }
-        vd = col_ok ? row[voff] : 0.0f;
-    };
-    if (T > 0) fetch(0, q, f, v);
-    for (int t = 0; t < T; ++t) {
-        float qn[kScanRows], fn[kScanRows], vn = 0.0f;
-        if (t + 1 < T) fetch(t + 1, qn, fn, vn);
-        float o = 0.0f;
-#pragma unroll
-        for (int r = 0; r < kScanRows; ++r) {
-            S[r] = fmaf(f[r], S[r], (1.0f - f[r]) * v);
-            o = fmaf(S[r], q[r], o);
+        for (int idx = threadIdx.x; idx < nb * cols; idx += blockDim.x) {
+            const int tt = idx / cols, jj = idx % cols;
+            sv[idx] = j0 + jj < V ? proj[(size_t)(m0 + tb + tt) * ld + 2 * HD + h * V + j0 + jj] : 0.0f;
         }
+        __syncthreads();
+        for (int tt = 0; tt < nb; ++tt) {
+            const f32x4* q4 = reinterpret_cast<const f32x4*>(sq + tt * Dp + g * kScanRows);
+            const f32x4* f4 = reinterpret_cast<const f32x4*>(sf + tt * Dp + g * kScanRows);
+            const float v = sv[tt * cols + jl];
+            float o = 0.0f;
 #pragma unroll
-        for (int off = 1; off < G; off <<= 1) o += __shfl_xor(o, off, 64);
-        if (g == 0 && col_ok) out[(size_t)(m0 + t) * ldo + h * V + j] = o;
-        if (t + 1 < T) {
+            for (int r4 = 0; r4 < kScanRows / 4; ++r4) {
+                const f32x4 qq = q4[r4], ff = f4[r4];
+                const float qv[4] = {qq.x, qq.y, qq.z, qq.w}, fv[4] = {ff.x, ff.y, ff.z, ff.w};
 #pragma unroll
-            for (int r = 0; r < kScanRows; ++r) {
-                q[r] = qn[r];
-                f[r] = fn[r];
+                for (int u = 0; u < 4; ++u) {
+                    const int r = r4 * 4 + u;
+                    S[r] = fmaf(fv[u], S[r], (1.0f - fv[u]) * v);
+                    o = fmaf(S[r], qv[u], o);
+                    if (mode == SCAN_A) A[r] *= fv[u];
+                }
             }
-            v = vn;
+            if (mode != SCAN_A) {
+#pragma unroll
+                for (int off = 1; off < G; off <<= 1) o += __shfl_xor(o, off, 64);
+                if (g == 0 && col_ok) out[(size_t)(m0 + tb + tt) * ldo + h * V + j] = o;
+            }
         }
     }
+    float* S_out = mode == SCAN_DIRECT ? S_slot : mode == SCAN_A ? S_ws : nullptr;
+    if (S_out) {
 #pragma unroll
-    for (int r = 0; r < kScanRows; ++r)
-        if (ok[r]) S_mem[(size_t)(g * kScanRows + r) * V + j] = S[r];
+        for (int r = 0; r < kScanRows; ++r) {
+            const int i = g * kScanRows + r;
+            if (col_ok && i < D) S_out[(size_t)i * V + j] = S[r];
+        }
+    }
+    if (mode == SCAN_A && blockIdx.z == 0 && jl == 0) {
+#pragma unroll
+        for (int r = 0; r < kScanRows; ++r) {
+            const int i = g * kScanRows + r;
+            if (i < D) wsA[((size_t)blockIdx.x * H + h) * D + i] = A[r];
+        }
+    }
+}
+
+// phase B: one thread per state element walks the chunks of its entry
+__global__ __launch_bounds__(256) void hgrn2_carry_kernel(float* state, size_t slot_stride, const int* ent_len, const int* ent_slot, int n_entries, int H,
+                                                          int D, int V, float* wsB, const float* wsA) {
+    const int e = blockIdx.y;
+    const size_t n = (size_t)H * D * V, idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= n) return;
+    int first = 0;
+    for (int k = 0; k < e; ++k) first += (ent_len[k] + kScanChunk - 1) / kScanChunk;
+    const int nc = (ent_len[e] + kScanChunk - 1) / kScanChunk;
+    const size_t hi = idx / V;  // (head, row)
+    float* slot = state + (size_t)ent_slot[e] * slot_stride;
+    float S = slot[idx];
+    for (int c = 0; c < nc; ++c) {
+        float* b = wsB + (size_t)(first + c) * n + idx;
+        const float B = *b, A = wsA[(size_t)(first + c) * H * D + hi];
+        *b = S;  // the chunk's start state for phase C
+        S = fmaf(A, S, B);
+    }
+    if (nc > 0) slot[idx] = S;
 }
 
 // ------------------------------------------------------------------------------------------------ latent attention
@@ -228,14 +309,23 @@ __global__ __launch_bounds__(256) void q_rotary_kernel(const float* q, int ldq, 
 
 // One workgroup per (row, head).  The lanes of a wave split the KR + R dimensions of a cache row (ND per lane); a wave walks
 // its share of the keys four at a time with a running (maximum, sum, weighted latent) and the four waves are merged at the end.
+// With n_split > 1 (decode steps: few rows, long key ranges) grid.z workgroups share a row's keys in ranges of at least 64
+// and leave (maximum, sum, weighted latent) partials in ws for latent_merge_kernel.
 template <int ND>
 __global__ __launch_bounds__(256) void latent_attention_kernel(const float* qa, float* ctx, int H, int KR, int R, float scale, const int* row_pos,
                                                                const int* row_slot, const int* page_table, int max_pages, int page_tokens,
-                                                               const float* cache) {
+                                                               const float* cache, float* ws, int n_split) {
     __shared__ float s_m[4], s_l[4];
     __shared__ float s_acc[4][ND * 64];
     const int m = blockIdx.x, h = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int DT = KR + R, n_keys = row_pos[m] + 1, slot = row_slot[m];
+    int k_lo = 0, k_hi = n_keys;
+    if (n_split > 1) {
+        int chunk = (n_keys + n_split - 1) / n_split;
+        chunk = max(64, (chunk + 15) & ~15);
+        k_lo = min(n_keys, (int)blockIdx.z * chunk);
+        k_hi = min(n_keys, k_lo + chunk);
+    }
     const float* qrow = qa + ((size_t)m * H + h) * DT;
     float q[ND], acc[ND];
 #pragma unroll
@@ -246,11 +336,11 @@ __global__ __launch_bounds__(256) void latent_attention_kernel(const float* qa, 
     }
     float mx = -INFINITY, l = 0.0f;
     const int* pt = page_table + (size_t)slot * max_pages;
-    for (int kb = wave * 4; kb < n_keys; kb += 16) {
+    for (int kb = k_lo + wave * 4; kb < k_hi; kb += 16) {
         float r[4][ND], s[4];
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
-            const int key = kb + u < n_keys ? kb + u : kb;
+            const int key = kb + u < k_hi ? kb + u : kb;
             const float* row = cache + ((size_t)pt[key / page_tokens] * page_tokens + key % page_tokens) * DT;
             float part = 0.0f;
 #pragma unroll
@@ -264,7 +354,7 @@ __global__ __launch_bounds__(256) void latent_attention_kernel(const float* qa, 
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             s[u] = wave_allsum(s[u]) * scale;
-            if (kb + u >= n_keys) s[u] = -INFINITY;
+            if (kb + u >= k_hi) s[u] = -INFINITY;
         }
         const float mn = fmaxf(fmaxf(mx, s[0]), fmaxf(fmaxf(s[1], s[2]), s[3]));
         const float alpha = expf(mx - mn);  // 0 for the first group (mx = -inf, mn finite: key kb is always valid)
@@ -292,8 +382,22 @@ __global__ __launch_bounds__(256) void latent_attention_kernel(const float* qa, 
     float wgt[4], L = 0.0f;
 #pragma unroll
     for (int w = 0; w < 4; ++w) {
-        wgt[w] = expf(s_m[w] - M4);  // a wave without keys: exp(-inf) = 0
+        wgt[w] = M4 == -INFINITY ? 0.0f : expf(s_m[w] - M4);  // a wave without keys: exp(-inf) = 0; a range without keys: all zero
         L += wgt[w] * s_l[w];
+    }
+    if (n_split > 1) {
+        float* part = ws + (((size_t)m * H + h) * n_split + blockIdx.z) * (KR + 2);
+        if (threadIdx.x == 0) {
+            part[0] = M4;
+            part[1] = L;
+        }
+        for (int d = threadIdx.x; d < KR; d += blockDim.x) {
+            float a = 0.0f;
+#pragma unroll
+            for (int w = 0; w < 4; ++w) a = fmaf(wgt[w], s_acc[w][d], a);
+            part[2 + d] = a;
+        }
+        return;
     }
     float* out = ctx + ((size_t)m * H + h) * KR;
     for (int d = threadIdx.x; d < KR; d += blockDim.x) {
@@ -304,17 +408,202 @@ __global__ __launch_bounds__(256) void latent_attention_kernel(const float* qa, 
     }
 }
 
-__global__ __launch_bounds__(256) void row_argmax_kernel(const float* logits, int n, float* max_out, int* idx_out) {
+// Prompt portions in bf16 mode: the same attention on the matrix cores.  A workgroup takes 32 consecutive queries of one entry
+// and four heads (one per wave) — the heads share the cached rows, so a tile of 32 keys is staged in the LDS once for all four:
+// as bf16 rows [key][dim] for the scores and, its latent part, transposed [dim][key] for the weighted sum.  Both products are
+// computed transposed (S^T = K Q^T, O^T = C^T P^T): a lane's column is a query, so the running maximum and sum are per-lane
+// values and the probabilities a lane computed are exactly the eight per k-step it has to feed back (in a key order that the
+// transposed latent tile is read in as well: keys {0-3, 8-11} from the lower half-wave, {4-7, 12-15} from the upper one).
+// Scores, softmax and both accumulations are fp32; q, cache rows and probabilities enter the products as bf16.
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+
+template <int NKS, int NT>  // 16 NKS >= KR + R (score dimensions), 32 NT >= KR (latent dimensions)
+__global__ __launch_bounds__(256) void latent_attention_mfma_kernel(const float* qa, float* ctx, int H, int KR, int R, float scale,
+                                                                    const int* ent_start, const int* ent_len, const int* ent_slot, int n_entries,
+                                                                    const int* row_pos, const int* page_table, int max_pages, int page_tokens,
+                                                                    const float* cache) {
+    constexpr int DTp = NKS * 16, KS_LD = DTp + 8, VT_LD = 40;
+    __shared__ __attribute__((aligned(16))) bf16_t Ks[32 * KS_LD];
+    __shared__ __attribute__((aligned(16))) bf16_t Vt[NT * 32 * VT_LD];
+    int id = blockIdx.x, e = 0, qb = 0;
+    for (; e < n_entries; ++e) {
+        const int nb = (ent_len[e] + 31) / 32;
+        if (id < nb) {
+            qb = id;
+            break;
+        }
+        id -= nb;
+    }
+    if (e >= n_entries) return;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, hf = lane >> 5;
+    const int h = blockIdx.y * 4 + wave;
+    const bool head_ok = h < H;
+    const int m_first = ent_start[e] + qb * 32, nq = min(32, ent_len[e] - qb * 32);
+    const int pos_first = row_pos[m_first], qpos = pos_first + r, DT = KR + R;
+    const bool q_ok = r < nq;
+    const int n_keys = pos_first + nq;
+    const int* pt = page_table + (size_t)ent_slot[e] * max_pages;
+
+    bf16x8 qf[NKS];
+    {
+        const float* qrow = qa + ((size_t)(m_first + (q_ok ? r : 0)) * H + (head_ok ? h : 0)) * DT;
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int d = ks * 16 + 8 * hf + u;
+                v[u] = (head_ok && q_ok && d < DT) ? qrow[d] : 0.0f;
+            }
+            u32x4 pk;
+            pk.x = cvt_pk_bf16(v[0], v[1]);
+            pk.y = cvt_pk_bf16(v[2], v[3]);
+            pk.z = cvt_pk_bf16(v[4], v[5]);
+            pk.w = cvt_pk_bf16(v[6], v[7]);
+            qf[ks] = __builtin_bit_cast(bf16x8, pk);
+        }
+    }
+    f32x16 o[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o[t][i] = 0.0f;
+    float mx = -INFINITY, lsum = 0.0f;
+    const bool vec = (DT % 4 == 0) && ((reinterpret_cast<uintptr_t>(cache) & 15) == 0);
+
+    for (int kt = 0; kt * 32 < n_keys; ++kt) {
+        __syncthreads();  // the previous tile has been consumed
+        for (int idx = tid; idx < 32 * (DTp / 4); idx += 256) {
+            const int key = idx / (DTp / 4), d4 = (idx % (DTp / 4)) * 4, kpos = kt * 32 + key;
+            float v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+            if (kpos < n_keys) {
+                const float* row = cache + ((size_t)pt[kpos / page_tokens] * page_tokens + kpos % page_tokens) * DT;
+                if (vec && d4 + 4 <= DT) {
+                    const f32x4 x = *reinterpret_cast<const f32x4*>(row + d4);
+                    v[0] = x.x; v[1] = x.y; v[2] = x.z; v[3] = x.w;
+                } else {
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) v[u] = d4 + u < DT ? row[d4 + u] : 0.0f;
+                }
+            }
+            u32x2 pk;
+            pk.x = cvt_pk_bf16(v[0], v[1]);
+            pk.y = cvt_pk_bf16(v[2], v[3]);
+            *reinterpret_cast<u32x2*>(&Ks[key * KS_LD + d4]) = pk;
+            if (d4 < NT * 32) {
+                Vt[(d4 + 0) * VT_LD + key] = (bf16_t)(pk.x & 0xFFFFu);
+                Vt[(d4 + 1) * VT_LD + key] = (bf16_t)(pk.x >> 16);
+                Vt[(d4 + 2) * VT_LD + key] = (bf16_t)(pk.y & 0xFFFFu);
+                Vt[(d4 + 3) * VT_LD + key] = (bf16_t)(pk.y >> 16);
+            }
+        }
+        __syncthreads();
+        if (!head_ok) continue;
+        f32x16 sacc;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) sacc[i] = 0.0f;
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) {
+            const bf16x8 a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(&Ks[r * KS_LD + ks * 16 + 8 * hf]));
+            sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[ks], sacc, 0, 0, 0);
+        }
+        float sv[16], tmax = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int key = kt * 32 + 8 * (i >> 2) + 4 * hf + (i & 3);
+            sv[i] = (q_ok && key <= qpos) ? sacc[i] * scale : -INFINITY;
+            tmax = fmaxf(tmax, sv[i]);
+        }
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+        const float mn = fmaxf(mx, tmax);
+        const bool none = mn == -INFINITY;  // a query row beyond the entry: nothing to weigh
+        const float alpha = none ? 1.0f : expf(mx - mn);
+        float psum = 0.0f, pv[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            pv[i] = none ? 0.0f : expf(sv[i] - mn);
+            psum += pv[i];
+        }
+        lsum = lsum * alpha + psum;
+        mx = mn;
+        u32x4 p0, p1;
+        p0.x = cvt_pk_bf16(pv[0], pv[1]); p0.y = cvt_pk_bf16(pv[2], pv[3]); p0.z = cvt_pk_bf16(pv[4], pv[5]); p0.w = cvt_pk_bf16(pv[6], pv[7]);
+        p1.x = cvt_pk_bf16(pv[8], pv[9]); p1.y = cvt_pk_bf16(pv[10], pv[11]); p1.z = cvt_pk_bf16(pv[12], pv[13]); p1.w = cvt_pk_bf16(pv[14], pv[15]);
+        const bf16x8 pf0 = __builtin_bit_cast(bf16x8, p0), pf1 = __builtin_bit_cast(bf16x8, p1);
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) o[t][i] *= alpha;
+            const bf16_t* vrow = &Vt[(t * 32 + r) * VT_LD + 4 * hf];
+            const u32x2 a0 = *reinterpret_cast<const u32x2*>(vrow), a1 = *reinterpret_cast<const u32x2*>(vrow + 8);
+            const u32x2 b0 = *reinterpret_cast<const u32x2*>(vrow + 16), b1 = *reinterpret_cast<const u32x2*>(vrow + 24);
+            o[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, (u32x4){a0.x, a0.y, a1.x, a1.y}), pf0, o[t], 0, 0, 0);
+            o[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, (u32x4){b0.x, b0.y, b1.x, b1.y}), pf1, o[t], 0, 0, 0);
+        }
+    }
+    if (!head_ok) return;
+    const float L = lsum + __shfl_xor(lsum, 32, 64);
+    if (!q_ok) return;
+    float* out = ctx + ((size_t)(m_first + r) * H + h) * KR;
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int d = t * 32 + 8 * (i >> 2) + 4 * hf + (i & 3);
+            if (d < KR) out[d] = o[t][i] / L;
+        }
+}
+
+// ctx[m][h] from the n_split partials of latent_attention_kernel (fixed order: the result does not depend on timing)
+__global__ __launch_bounds__(256) void latent_merge_kernel(const float* ws, float* ctx, int H, int KR, int n_split) {
+    const int m = blockIdx.x, h = blockIdx.y;
+    const float* part = ws + ((size_t)m * H + h) * n_split * (KR + 2);
+    float M = -INFINITY;
+    for (int sidx = 0; sidx < n_split; ++sidx) M = fmaxf(M, part[(size_t)sidx * (KR + 2)]);
+    float L = 0.0f;
+    for (int sidx = 0; sidx < n_split; ++sidx) {
+        const float pm = part[(size_t)sidx * (KR + 2)];
+        if (pm != -INFINITY) L += expf(pm - M) * part[(size_t)sidx * (KR + 2) + 1];
+    }
+    float* out = ctx + ((size_t)m * H + h) * KR;
+    for (int d = threadIdx.x; d < KR; d += blockDim.x) {
+        float a = 0.0f;
+        for (int sidx = 0; sidx < n_split; ++sidx) {
+            const float pm = part[(size_t)sidx * (KR + 2)];
+            if (pm != -INFINITY) a = fmaf(expf(pm - M), part[(size_t)sidx * (KR + 2) + 2 + d], a);
+        }
+        out[d] = a / L;
+    }
+}
+
+// Stage 1: block (row, part) finds the maximum and its first index in its slice of the row; stage 2 (parts == 1 in the grid,
+// n_parts > 0 as argument): one block per row combines the parts.  The first maximum wins; a row of NaNs gives index 0.
+__global__ __launch_bounds__(256) void row_argmax_kernel(const float* logits, int n, float* max_out, int* idx_out, float* part_val, int* part_idx,
+                                                         int n_parts, int combine) {
     __shared__ float s_v[4];
     __shared__ int s_i[4];
-    const float* row = logits + (size_t)blockIdx.x * n;
+    const int row = blockIdx.x;
     float best = -INFINITY;
     int bi = 0x7fffffff;
-    for (int i = threadIdx.x; i < n; i += blockDim.x) {
-        const float v = row[i];
-        if (v > best) {  // ascending i per thread: the first maximum stays
-            best = v;
-            bi = i;
+    if (!combine) {
+        const int per = (n + n_parts - 1) / n_parts, lo = blockIdx.y * per, hi = min(n, lo + per);
+        const float* r = logits + (size_t)row * n;
+        for (int i = lo + threadIdx.x; i < hi; i += blockDim.x) {
+            const float v = r[i];
+            if (v > best) {  // ascending i per thread: the first maximum stays
+                best = v;
+                bi = i;
+            }
+        }
+    } else {
+        for (int i = threadIdx.x; i < n_parts; i += blockDim.x) {
+            const float v = part_val[(size_t)row * n_parts + i];
+            const int ix = part_idx[(size_t)row * n_parts + i];
+            if (v > best || (v == best && ix < bi)) {
+                best = v;
+                bi = ix;
+            }
         }
     }
     const float wbest = wave_allmax(best);
@@ -335,9 +624,14 @@ __global__ __launch_bounds__(256) void row_argmax_kernel(const float* logits, in
                 v = s_v[w];
                 ix = s_i[w];
             }
-        if (ix == 0x7fffffff) ix = 0;  // a row of NaNs
-        if (max_out) max_out[blockIdx.x] = v;
-        if (idx_out) idx_out[blockIdx.x] = ix;
+        if (!combine) {
+            part_val[(size_t)row * n_parts + blockIdx.y] = v;
+            part_idx[(size_t)row * n_parts + blockIdx.y] = ix;
+        } else {
+            if (ix == 0x7fffffff) ix = 0;
+            if (max_out) max_out[row] = v;
+            if (idx_out) idx_out[row] = ix;
+        }
     }
 }
 
@@ -398,25 +692,49 @@ int launch_hgrn2_gates(float* proj, int ld, int M, int HD, const float* bias, co
 }
 
 int launch_hgrn2_scan(const float* proj, int ld, float* out, int ldo, float* state, size_t slot_stride, const int* ent_start,
-                      const int* ent_len, const int* ent_slot, int n_entries, int H, int D, int V, hipStream_t s) {
+                      const int* ent_len, const int* ent_slot, int n_entries, int M, int H, int D, int V, float* ws, size_t ws_floats,
+                      hipStream_t s) {
     if (n_entries <= 0) return ZG_OK;
     ZG_REQUIRE(D >= 1 && D <= 16 * kScanRows, ZG_ERR_UNSUPPORTED, "hgrn2: %d key channels per head (at most %d)", D, 16 * kScanRows);
     int G = 1;
     while (G * kScanRows < D) G <<= 1;
+    const int Dp = G * kScanRows;
     int threads = ((V * G + 63) / 64) * 64;
     if (threads > 256) threads = 256;
     const int cols = threads / G;
-    const dim3 grid(n_entries, H, (V + cols - 1) / cols);
-#define ZG_SCAN(G_) hgrn2_scan_kernel<G_><<<grid, threads, 0, s>>>(proj, ld, out, ldo, state, slot_stride, ent_start, ent_len, ent_slot, H, D, V)
-    switch (G) {
-        case 1: ZG_SCAN(1); break;
-        case 2: ZG_SCAN(2); break;
-        case 4: ZG_SCAN(4); break;
-        case 8: ZG_SCAN(8); break;
-        default: ZG_SCAN(16); break;
+    const int SB = std::max(1, std::min(kScanChunk, std::min(4096 / Dp, 8192 / cols)));
+    const size_t lds = ((size_t)2 * SB * Dp + (size_t)SB * cols) * sizeof(float);
+    // chunked when the step is long enough to pay for two passes, and the workspace holds every chunk's state
+    const int max_chunks = (M + kScanChunk - 1) / kScanChunk + n_entries;
+    const size_t head_floats = (size_t)H * D * V, need = (size_t)max_chunks * (head_floats + (size_t)H * D);
+    const bool chunked = M >= 4 * kScanChunk && ws && ws_floats >= need;
+    float* wsB = chunked ? ws : nullptr;
+    float* wsA = chunked ? ws + (size_t)max_chunks * head_floats : nullptr;
+#define ZG_SCAN(G_, grid_x, mode)                                                                                                                 \
+    hgrn2_scan_kernel<G_><<<dim3(grid_x, H, (V + cols - 1) / cols), threads, lds, s>>>(proj, ld, out, ldo, state, slot_stride, ent_start, ent_len, \
+                                                                                        ent_slot, n_entries, H, D, V, mode, SB, wsB, wsA)
+#define ZG_SCAN_G(grid_x, mode)                    \
+    switch (G) {                                   \
+        case 1: ZG_SCAN(1, grid_x, mode); break;   \
+        case 2: ZG_SCAN(2, grid_x, mode); break;   \
+        case 4: ZG_SCAN(4, grid_x, mode); break;   \
+        case 8: ZG_SCAN(8, grid_x, mode); break;   \
+        default: ZG_SCAN(16, grid_x, mode); break; \
     }
-#undef ZG_SCAN
+    if (!chunked) {
+        ZG_SCAN_G(n_entries, SCAN_DIRECT);
+        ZG_HIP(hipGetLastError());
+        return ZG_OK;
+    }
+    ZG_SCAN_G(max_chunks, SCAN_A);
     ZG_HIP(hipGetLastError());
+    hgrn2_carry_kernel<<<dim3((unsigned)((head_floats + 255) / 256), n_entries), 256, 0, s>>>(state, slot_stride, ent_len, ent_slot, n_entries, H, D, V,
+                                                                                                wsB, wsA);
+    ZG_HIP(hipGetLastError());
+    ZG_SCAN_G(max_chunks, SCAN_C);
+    ZG_HIP(hipGetLastError());
+#undef ZG_SCAN_G
+#undef ZG_SCAN
     return ZG_OK;
 }
 
@@ -439,15 +757,41 @@ int launch_q_rotary(const float* q, int ldq, float* qa, int ldqa, int M, int H, 
     return ZG_OK;
 }
 
+int launch_latent_attention_tiles(const float* qa, float* ctx, int M, int H, int KR, int R, float scale, const int* ent_start, const int* ent_len,
+                                  const int* ent_slot, int n_entries, const int* row_pos, const int* page_table, int max_pages, int page_tokens,
+                                  const float* cache, hipStream_t s, bool* taken) {
+    *taken = false;
+    if (M <= 0 || n_entries <= 0) return ZG_OK;
+    const int DT = KR + R;
+    const dim3 grid((M + 31) / 32 + n_entries, (H + 3) / 4);
+#define ZG_ATT_T(NKS_, NT_)                                                                                                                      \
+    latent_attention_mfma_kernel<NKS_, NT_><<<grid, 256, 0, s>>>(qa, ctx, H, KR, R, scale, ent_start, ent_len, ent_slot, n_entries, row_pos, page_table, \
+                                                                 max_pages, page_tokens, cache)
+    if (DT <= 96 && KR <= 64) ZG_ATT_T(6, 2);
+    else if (DT <= 160 && KR <= 128) ZG_ATT_T(10, 4);
+    else if (DT <= 288 && KR <= 256) ZG_ATT_T(18, 8);
+    else if (DT <= 384 && KR <= 320) ZG_ATT_T(24, 10);
+    else return ZG_OK;  // larger latents: the caller's general kernel
+#undef ZG_ATT_T
+    ZG_HIP(hipGetLastError());
+    *taken = true;
+    return ZG_OK;
+}
+
 int launch_latent_attention(const float* qa, float* ctx, int M, int H, int KR, int R, float scale, const int* row_pos, const int* row_slot,
                             const int* page_table, int max_pages, int page_tokens, const float* cache, float* ws, size_t ws_floats,
                             hipStream_t s) {
     if (M <= 0) return ZG_OK;
     const int nd = (KR + R + 63) / 64;
     ZG_REQUIRE(nd <= 16, ZG_ERR_UNSUPPORTED, "latent attention: %d cached dimensions per token (at most 1024)", KR + R);
-    const dim3 grid(M, H);
-#define ZG_ATT(ND_) \
-    latent_attention_kernel<ND_><<<grid, 256, 0, s>>>(qa, ctx, H, KR, R, scale, row_pos, row_slot, page_table, max_pages, page_tokens, cache)
+    // decode steps: the keys of a row in up to kAttnSplits ranges (a fixed grid, so that a captured step can be replayed at any
+    // sequence length; ranges beyond the row's keys leave empty partials)
+    int n_split = 1;
+    if (M <= kGemvMaxRows && ws && ws_floats >= (size_t)M * H * kAttnSplits * (KR + 2) && (long long)max_pages * page_tokens > 128) n_split = kAttnSplits;
+    const dim3 grid(M, H, n_split);
+#define ZG_ATT(ND_)                                                                                                                           \
+    latent_attention_kernel<ND_><<<grid, 256, 0, s>>>(qa, ctx, H, KR, R, scale, row_pos, row_slot, page_table, max_pages, page_tokens, cache, ws, \
+                                                      n_split)
     if (nd <= 1) ZG_ATT(1);
     else if (nd <= 2) ZG_ATT(2);
     else if (nd <= 3) ZG_ATT(3);
@@ -458,12 +802,19 @@ int launch_latent_attention(const float* qa, float* ctx, int M, int H, int KR, i
     else ZG_ATT(16);
 #undef ZG_ATT
     ZG_HIP(hipGetLastError());
+    if (n_split > 1) {
+        latent_merge_kernel<<<dim3(M, H), 256, 0, s>>>(ws, ctx, H, KR, n_split);
+        ZG_HIP(hipGetLastError());
+    }
     return ZG_OK;
 }
 
-int launch_row_argmax(const float* logits, int rows, int n, float* max_out, int* idx_out, hipStream_t s) {
+int launch_row_argmax(const float* logits, int rows, int n, float* max_out, int* idx_out, float* part_val, int* part_idx, hipStream_t s) {
     if (rows <= 0) return ZG_OK;
-    row_argmax_kernel<<<rows, 256, 0, s>>>(logits, n, max_out, idx_out);
+    const int parts = std::max(1, std::min(kArgmaxParts, (n + 1023) / 1024));
+    row_argmax_kernel<<<dim3(rows, parts), 256, 0, s>>>(logits, n, nullptr, nullptr, part_val, part_idx, parts, 0);
+    ZG_HIP(hipGetLastError());
+    row_argmax_kernel<<<dim3(rows, 1), 256, 0, s>>>(logits, n, max_out, idx_out, part_val, part_idx, parts, 1);
     ZG_HIP(hipGetLastError());
     return ZG_OK;
 }

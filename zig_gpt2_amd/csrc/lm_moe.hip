@@ -23,7 +23,8 @@ __device__ __forceinline__ float block_allsum(float v, float* s_red) {
     return t;
 }
 
-// one wave per row; lane l scores the experts l, l + 64, l + 128, l + 192
+// one wave per row: the lanes split the row's W channels (four at a time), a router row is one dot product summed over the
+// wave; lane e % 64 keeps the logit of expert e (experts e, e + 64, e + 128, e + 192 in its four slots)
 __global__ __launch_bounds__(256) void route_kernel(const float* g, int M, int W, const bf16_t* router, const float* correction, int E, int top,
                                                     int* pick, float* weight) {
     const int m = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
@@ -31,14 +32,28 @@ __global__ __launch_bounds__(256) void route_kernel(const float* g, int M, int W
     const float* row = g + (size_t)m * W;
     float z[4], sc[4], ch[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int e = lane + 64 * i;
-        z[i] = -INFINITY;
-        if (e < E) {
-            const bf16_t* wr = router + (size_t)e * W;
-            float a = 0.0f;
-            for (int k = 0; k < W; ++k) a = fmaf(row[k], __uint_as_float((uint32_t)wr[k] << 16), a);
-            z[i] = a;
+    for (int i = 0; i < 4; ++i) z[i] = -INFINITY;
+    const bool vec = (W % 4 == 0) && ((reinterpret_cast<uintptr_t>(g) & 15) == 0) && ((reinterpret_cast<uintptr_t>(router) & 7) == 0);
+    for (int e = 0; e < E; ++e) {
+        const bf16_t* wr = router + (size_t)e * W;
+        float a = 0.0f;
+        if (vec) {
+            for (int k = lane * 4; k < W; k += 256) {
+                const f32x4 x = *reinterpret_cast<const f32x4*>(row + k);
+                const u32x2 w2 = *reinterpret_cast<const u32x2*>(wr + k);
+                a = fmaf(x.x, bf16_lo(w2.x), a);
+                a = fmaf(x.y, bf16_hi(w2.x), a);
+                a = fmaf(x.z, bf16_lo(w2.y), a);
+                a = fmaf(x.w, bf16_hi(w2.y), a);
+            }
+        } else {
+            for (int k = lane; k < W; k += 64) a = fmaf(row[k], __uint_as_float((uint32_t)wr[k] << 16), a);
+        }
+        a = wave_allsum(a);
+        if ((e & 63) == lane) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if ((e >> 6) == i) z[i] = a;
         }
     }
     const float mx = wave_allmax(fmaxf(fmaxf(z[0], z[1]), fmaxf(z[2], z[3])));

@@ -155,7 +155,7 @@ class LayeredLM:
     """A handle of the layered-model tier: weights, state slots, the step function and generation."""
 
     def __init__(self, config: LMConfig, dtype="bfloat16", max_tokens=4096, max_seqs=8, max_step_tokens=0, page_tokens=0, device=0,
-                 build_if_missing=False):
+                 build_if_missing=False, use_graph=True):
         if dtype not in ("bfloat16", "float32"):
             raise ValueError(f"dtype {dtype!r}: bfloat16 or float32")
         self.config, self.dtype = config, dtype
@@ -163,7 +163,8 @@ class LayeredLM:
         self._layers = (_lib.LmLayer * len(config.layers))(*[l.to_c() for l in config.layers])
         loop = config.loop or {"start": 0, "stop": 0, "times": 1}
         cfg = _lib.LmConfig(config.vocab, config.width, len(config.layers), self._layers, int(loop["start"]), int(loop["stop"]), int(loop["times"]),
-                            config.norm_eps, max_tokens, max_seqs, max_step_tokens, page_tokens, _lib.LM_F32 if dtype == "float32" else 0)
+                            config.norm_eps, max_tokens, max_seqs, max_step_tokens, page_tokens,
+                            (_lib.LM_F32 if dtype == "float32" else 0) | (0 if use_graph else _lib.LM_NO_GRAPH))
         h = C.c_void_p()
         check(L.zg_lm_create(C.byref(h), C.byref(cfg), device))
         self.h = h
