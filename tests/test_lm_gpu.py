@@ -48,6 +48,7 @@ SINGLE = {
     "moe": [tl.hgrn2_layer(mlp=tl.moe_mlp())],
     "moe_top1": [tl.hgrn2_layer(mlp=tl.moe_mlp(ff=20, experts=3, top=1))],
     "moe_all": [tl.hgrn2_layer(mlp=tl.moe_mlp(ff=8, experts=4, top=4))],
+    "moe_many": [tl.hgrn2_layer(mlp=tl.moe_mlp(ff=8, experts=70, top=3))],  # more experts than a wave has lanes
 }
 
 
@@ -254,6 +255,20 @@ def test_larger_odd_sizes_take_the_tiled_products():
         m.close()
 
 
+def test_large_tiles_on_small_shapes(monkeypatch):
+    """The 128 x 128 tiles (taken by themselves only from thousands of rows) on shapes with ragged edges, grouped products included."""
+    monkeypatch.setenv("ZGPT2_LM_GEMM_TILE", "128")
+    cfg = tl.config([tl.hgrn2_layer(heads=3, dim=20, vdim=28, mlp=tl.moe_mlp(ff=36, experts=3, top=2)),
+                     tl.latent_layer(heads=2, dim=12, vdim=20, rot_dim=6, kv_rank=52, q_rank=44, mlp=tl.dense_mlp(ff=150))], vocab=203, width=76)
+    w = tl.weights(cfg, seed=17)
+    toks = tl.tokens(62, 300, cfg["vocab"])
+    ref = lm_oracle.Model(cfg, w).forward(toks)[0]
+    for dtype in ("float32", "bfloat16"):
+        m = make(cfg, w, dtype)
+        tl.assert_close(run_whole(m, toks), ref, dtype, dtype)
+        m.close()
+
+
 def test_greedy_and_sampled_generation():
     cfg = full_cfg(loop={"start": 1, "stop": 3, "times": 2})
     w = tl.weights(cfg, seed=14, head_std=1.0)
@@ -305,3 +320,69 @@ def test_errors_are_reported():
     bad["layers"][1]["mixer"]["rot"]["dims"] = 7
     with pytest.raises(Exception):
         lm.LayeredLM(lm.LMConfig.from_json(bad), max_tokens=64)
+
+
+def _checkpoint(tmp_path, cfg, w):
+    import json
+
+    from zig_gpt2_amd import weights_io
+
+    d = tmp_path / "ckpt"
+    d.mkdir()
+    (d / "config.json").write_text(json.dumps(cfg))
+    weights_io.write_safetensors(str(d / "model.safetensors"), w)
+    return str(d)
+
+
+def test_checkpoint_folder_through_registry_host_program_and_trace_replay(tmp_path):
+    """One checkpoint folder, three front ends: models.load_model (the registry picks the class from config.json), the C++ host
+    program's `lm` command, and the trace replay program — all on the library's step / generate."""
+    import json
+    import os
+    import subprocess
+    import sys
+
+    from zig_gpt2_amd import models
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    cfg = full_cfg(loop={"start": 1, "stop": 3, "times": 2})
+    w = tl.weights(cfg, seed=16, head_std=1.0)
+    path = _checkpoint(tmp_path, cfg, w)
+    prompts = [tl.tokens(80, 11, cfg["vocab"]), tl.tokens(81, 4, cfg["vocab"])]
+    m = models.load_model(path, dtype="float32", max_tokens=256, max_seqs=4)
+    assert isinstance(m, lm.LayeredLM)
+    want = m.generate(prompts, 9)
+    ref = lm_oracle.Model(cfg, w).forward(prompts[0])[0]
+    s = m.open()
+    tl.assert_close(m.step([(s, prompts[0], list(range(11)))]), ref, "float32")
+    m.close()
+    exe = os.path.join(root, "zig_gpt2_amd", "bin", "zgpt2_main")
+    arg = ";".join(",".join(str(int(t)) for t in p) for p in prompts)
+    out = subprocess.run([exe, "lm", path, arg, "9", "--dtype", "float32"], capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0, out.stderr
+    got = np.array([[int(t) for t in line.split()] for line in out.stdout.strip().splitlines()])
+    assert np.array_equal(got, want)
+    bad = subprocess.run([exe, "lm", path, "1,100000", "2"], capture_output=True, text=True, timeout=120)
+    assert bad.returncode != 0 and "vocabulary" in bad.stderr
+    # trace replay: a prompt in two portions and two decoded tokens, a second request between them, the first one ended and its
+    # slot taken again
+    a, b = [int(t) for t in prompts[0]], [int(t) for t in prompts[1]]
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": a[:6], "want": [5]}], "end": []},
+             {"step": 1, "entries": [{"id": "a", "tokens": a[6:9], "want": []}], "end": []},
+             {"step": 2, "entries": [{"id": "b", "tokens": b, "want": [0, 3]}], "end": ["b"]},
+             {"step": 3, "entries": [{"id": "a", "tokens": a[9:10], "want": [0]}], "end": []},
+             {"step": 4, "entries": [{"id": "a", "tokens": a[10:11], "want": [0]}], "end": ["a"]},
+             {"step": 5, "entries": [{"id": "c", "tokens": a, "want": [10]}], "end": ["c"]}]
+    outdir = tmp_path / "out"
+    run = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", path, "--dtype", "float32", "--out", str(outdir),
+                          "--max-tokens", "64"], input="\n".join(json.dumps(x) for x in steps) + "\n", capture_output=True, text=True, timeout=300)
+    assert run.returncode == 0, run.stderr
+    assert [l for l in run.stdout.splitlines() if l.startswith("done")] == [f"done {i}" for i in range(6)]
+    refb = lm_oracle.Model(cfg, w).forward(prompts[1])[0]
+    rd = lambda i: np.fromfile(str(outdir / f"{i}.f32"), dtype="<f4").reshape(-1, cfg["vocab"])  # noqa: E731
+    assert not (outdir / "1.f32").exists()
+    tl.assert_close(rd(0), ref[5:6], "float32")
+    tl.assert_close(rd(2), refb[[0, 3]], "float32")
+    tl.assert_close(rd(3), ref[9:10], "float32")
+    tl.assert_close(rd(4), ref[10:11], "float32")
+    tl.assert_close(rd(5), ref[10:11], "float32")

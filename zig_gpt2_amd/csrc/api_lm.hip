@@ -397,9 +397,8 @@ int enqueue_layers(zg_lm* g, int M, int n_ent, bool capturing) {
             lin = Linear();
             lin.A = g->h; lin.lda = W; lin.B = L.qfv; lin.ldb = W; lin.C = g->proj; lin.ldc = NP; lin.M = M; lin.N = NP; lin.K = W;
             ZG_TRY(launch_linear(lin, f32, s));
-            ZG_TRY(launch_hgrn2_gates(g->proj, NP, M, HD, L.fb, L.lower, s));
             ZG_TRY(launch_hgrn2_scan(g->proj, NP, g->o, HV, g->hgrn_state + ps.hgrn_off, g->hgrn_floats, d_estart, d_elen, d_eslot, n_ent, M, H, D, Vd,
-                                     g->scan_ws, g->scan_ws_floats, s));
+                                     L.fb, L.lower, g->scan_ws, g->scan_ws_floats, s));
             ZG_TRY(launch_norm_plain(g->o, HV, H, Vd, M, L.hnorm, eps, s));
             lin = Linear();
             lin.A = g->o; lin.lda = HV; lin.B = L.o; lin.ldb = HV; lin.C = g->y; lin.ldc = W; lin.M = M; lin.N = W; lin.K = HV;
@@ -435,9 +434,8 @@ int enqueue_layers(zg_lm* g, int M, int n_ent, bool capturing) {
             lin.A = g->o; lin.lda = HV; lin.B = L.o; lin.ldb = HV; lin.C = g->y; lin.ldc = W; lin.M = M; lin.N = W; lin.K = HV;
             ZG_TRY(launch_linear(lin, f32, s));
         }
-        ZG_TRY(launch_norm_add(g->x, g->y, L.norm1b, eps, M, W, s));
-        if (d.ff != ZG_LM_FF_NONE)
-            ZG_TRY(launch_norm_shift(g->x, L.norm2, nullptr, eps, g->h, M, W, nullptr, nullptr, nullptr, 0, nullptr, nullptr, s));
+        if (d.ff != ZG_LM_FF_NONE) ZG_TRY(launch_norm_add_norm(g->x, g->y, L.norm1b, L.norm2, eps, g->h, M, W, s));
+        else ZG_TRY(launch_norm_add(g->x, g->y, L.norm1b, eps, M, W, s));
         const int F = d.ff_width;
         if (d.ff == ZG_LM_FF_DENSE) {
             lin = Linear();
@@ -462,7 +460,11 @@ int enqueue_layers(zg_lm* g, int M, int n_ent, bool capturing) {
                 up.M = dn.M = NA; up.a_rows = g->sorted; up.grp_off = dn.grp_off = g->grp_off; up.n_groups = dn.n_groups = E;
             }
             ZG_TRY(launch_linear(up, f32, s));
-            ZG_TRY(launch_glu(g->gu_buf, g->hb, NA, F, s));
+            if (few) {  // the gated activation is applied where the second product reads its rows
+                dn.A = g->gu_buf; dn.lda = 2 * F; dn.a_glu = F;
+            } else {
+                ZG_TRY(launch_glu(g->gu_buf, g->hb, NA, F, s));
+            }
             ZG_TRY(launch_linear(dn, f32, s));
             ZG_TRY(launch_moe_combine(g->x, g->ye, few ? nullptr : g->inv, g->wt, top, L.norm2b, eps, M, W, s));
         }

@@ -34,6 +34,7 @@ struct Linear {
     int ldc = 0;
     int M = 0, N = 0, K = 0;
     int act = ACT_NONE;
+    int a_glu = 0;  // > 0 (row-vector kernel only): A rows are [gate (a_glu) | up (a_glu)] and enter as silu(gate) * up, K = a_glu
     int nz = 1;
     long long a_zoff = 0, b_zoff = 0, c_zoff = 0;
     const int* z_group = nullptr;
@@ -61,21 +62,22 @@ int launch_commit_rows(float* dst, size_t slot_stride, const float* src, size_t 
                        int n_sets, size_t dst_set_stride, size_t src_set_stride, hipStream_t s);
 // x[m] += y[m] / rms(y[m]) * (1 + w)            (the norm behind a sublayer, then the residual sum)
 int launch_norm_add(float* x, const float* y, const float* w, float eps, int M, int W, hipStream_t s);
+// x[m] += y[m] / rms(y[m]) * (1 + wb);  h[m] = x[m] / rms(x[m]) * (1 + wn)   (the two above in one launch)
+int launch_norm_add_norm(float* x, const float* y, const float* wb, const float* wn, float eps, float* h, int M, int W, hipStream_t s);
 // out[j] = x[rows[j]] / rms * (1 + w)            (the model's last norm on the rows whose logits are asked for)
 int launch_norm_gather(const float* x, const int* rows, const float* w, float eps, float* out, int n_rows, int W, hipStream_t s);
 // In place over `rows` rows of `width` floats with row stride ld: v / rms(v) * w  (a plain weight; per-head norms)
 int launch_norm_plain(float* v, int ld, int rows_per_m, int width, int M, const float* w, float eps, hipStream_t s);
 
 // ------------------------------------------------------------------------------------------------ gated linear recurrence (HGRN2)
-// proj rows are [q (H D) | f (H D) | v (H V)] as the fused projection left them.  Activates in place:
-//   q <- silu(q);   f <- low + (1 - low) * sigmoid(f + bias)
-int launch_hgrn2_gates(float* proj, int ld, int M, int HD, const float* bias, const float* low, hipStream_t s);
+// proj rows are [q (H D) | f (H D) | v (H V)] as the fused projection left them; the gates are activated where the scan stages
+// them:  q <- silu(q);   f <- low + (1 - low) * sigmoid(f + bias)
 // Per entry e (rows ent_start[e] .. + ent_len[e]) and head: S <- diag(f_t) S + (1 - f_t) v_t^T, o_t = S^T q_t, token by token,
 // S = state[ent_slot[e]] ([H][D][V] fp32) read at the start and written back at the end.  out rows [H V], row stride ldo.
 // M: rows of the step.  ws (may be null): workspace for the chunk-parallel form of long steps, (M / 64 + n_entries) * (H D V + H D) floats.
 int launch_hgrn2_scan(const float* proj, int ld, float* out, int ldo, float* state, size_t slot_stride, const int* ent_start,
-                      const int* ent_len, const int* ent_slot, int n_entries, int M, int H, int D, int V, float* ws, size_t ws_floats,
-                      hipStream_t s);
+                      const int* ent_len, const int* ent_slot, int n_entries, int M, int H, int D, int V, const float* bias, const float* low,
+                      float* ws, size_t ws_floats, hipStream_t s);
 
 // ------------------------------------------------------------------------------------------------ latent attention
 // Rotary table of one layer: freq[i] for the rot_dims / 2 pairs (YaRN blend applied on the host) and the amplitude factor.

@@ -9,6 +9,8 @@
 //                      v_mfma_f32_32x32x2_f32.  Any M, N, K: tiles are zero-filled at the edges.
 // Both understand the same addressing: a row gather for A, one matrix per grid.z batch (heads), a matrix chosen per batch by
 // an index array (the expert of an assignment), and row groups sorted by expert with their offsets in device memory.
+#include <stdlib.h>
+
 #include <type_traits>
 
 #include "lm_kernels.h"
@@ -31,7 +33,7 @@ struct LinArgs {
     long long a_zoff, b_zoff, c_zoff;
     int lda, ldb, ldc;
     int M, N, K;
-    int a_div, act, n_groups;
+    int a_div, act, n_groups, a_glu;
     int a_vec, b_vec;  // 16-byte loads allowed (alignment of base, leading dimension and batch offsets)
 };
 
@@ -91,22 +93,46 @@ __global__ __launch_bounds__(256) void lm_gemv_kernel(const LinArgs p) {
     float acc0[MR], acc1[MR];
 #pragma unroll
     for (int m = 0; m < MR; ++m) acc0[m] = acc1[m] = 0.0f;
-    for (int k = lane * 8; k < p.K; k += 512) {
-        float wa[8], wb[8];
-        load_w8(w0, k, p.K, p.b_vec, wa);
-        load_w8(w1, k, p.K, p.b_vec, wb);
+    // two K pieces per trip, all four weight vectors requested before the first is used: rows of up to 1024 columns cost one
+    // memory round trip
+    for (int k = lane * 8; k < p.K; k += 1024) {
+        float wa[2][8], wb[2][8];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            load_w8(w0, k + 512 * u, p.K, p.b_vec, wa[u]);
+            load_w8(w1, k + 512 * u, p.K, p.b_vec, wb[u]);
+        }
 #pragma unroll
         for (int m = 0; m < MR; ++m) {
-            const f32x4 a0 = load_a4(arow[m], k, p.K, p.a_vec), a1 = load_a4(arow[m], k + 4, p.K, p.a_vec);
+            f32x4 av[2][2];
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                const int kk = k + 512 * u;
+                f32x4 a0 = load_a4(arow[m], kk, p.K, p.a_vec), a1 = load_a4(arow[m], kk + 4, p.K, p.a_vec);
+                if (p.a_glu > 0 && arow[m]) {  // rows [gate | up]: silu(gate) * up
+                    const f32x4 u0 = load_a4(arow[m] + p.a_glu, kk, p.K, p.a_vec && p.a_glu % 4 == 0);
+                    const f32x4 u1 = load_a4(arow[m] + p.a_glu, kk + 4, p.K, p.a_vec && p.a_glu % 4 == 0);
+                    a0.x = a0.x / (1.0f + expf(-a0.x)) * u0.x; a0.y = a0.y / (1.0f + expf(-a0.y)) * u0.y;
+                    a0.z = a0.z / (1.0f + expf(-a0.z)) * u0.z; a0.w = a0.w / (1.0f + expf(-a0.w)) * u0.w;
+                    a1.x = a1.x / (1.0f + expf(-a1.x)) * u1.x; a1.y = a1.y / (1.0f + expf(-a1.y)) * u1.y;
+                    a1.z = a1.z / (1.0f + expf(-a1.z)) * u1.z; a1.w = a1.w / (1.0f + expf(-a1.w)) * u1.w;
+                }
+                av[u][0] = a0;
+                av[u][1] = a1;
+            }
             float s0 = acc0[m], s1 = acc1[m];
-            s0 = fmaf(a0.x, wa[0], s0); s1 = fmaf(a0.x, wb[0], s1);
-            s0 = fmaf(a0.y, wa[1], s0); s1 = fmaf(a0.y, wb[1], s1);
-            s0 = fmaf(a0.z, wa[2], s0); s1 = fmaf(a0.z, wb[2], s1);
-            s0 = fmaf(a0.w, wa[3], s0); s1 = fmaf(a0.w, wb[3], s1);
-            s0 = fmaf(a1.x, wa[4], s0); s1 = fmaf(a1.x, wb[4], s1);
-            s0 = fmaf(a1.y, wa[5], s0); s1 = fmaf(a1.y, wb[5], s1);
-            s0 = fmaf(a1.z, wa[6], s0); s1 = fmaf(a1.z, wb[6], s1);
-            s0 = fmaf(a1.w, wa[7], s0); s1 = fmaf(a1.w, wb[7], s1);
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                const f32x4 a0 = av[u][0], a1 = av[u][1];
+                s0 = fmaf(a0.x, wa[u][0], s0); s1 = fmaf(a0.x, wb[u][0], s1);
+                s0 = fmaf(a0.y, wa[u][1], s0); s1 = fmaf(a0.y, wb[u][1], s1);
+                s0 = fmaf(a0.z, wa[u][2], s0); s1 = fmaf(a0.z, wb[u][2], s1);
+                s0 = fmaf(a0.w, wa[u][3], s0); s1 = fmaf(a0.w, wb[u][3], s1);
+                s0 = fmaf(a1.x, wa[u][4], s0); s1 = fmaf(a1.x, wb[u][4], s1);
+                s0 = fmaf(a1.y, wa[u][5], s0); s1 = fmaf(a1.y, wb[u][5], s1);
+                s0 = fmaf(a1.z, wa[u][6], s0); s1 = fmaf(a1.z, wb[u][6], s1);
+                s0 = fmaf(a1.w, wa[u][7], s0); s1 = fmaf(a1.w, wb[u][7], s1);
+            }
             acc0[m] = s0;
             acc1[m] = s1;
         }
@@ -312,7 +338,7 @@ int launch_linear(const Linear& L, bool f32, hipStream_t s) {
     p.A = L.A; p.B = L.B; p.C = L.C; p.a_rows = L.a_rows; p.z_group = L.z_group; p.grp_off = L.grp_off;
     p.a_zoff = L.a_zoff; p.b_zoff = L.b_zoff; p.c_zoff = L.c_zoff;
     p.lda = L.lda; p.ldb = L.ldb; p.ldc = L.ldc; p.M = L.M; p.N = L.N; p.K = L.K;
-    p.a_div = L.a_div; p.act = L.act; p.n_groups = L.grp_off ? L.n_groups : 0;
+    p.a_div = L.a_div; p.act = L.act; p.n_groups = L.grp_off ? L.n_groups : 0; p.a_glu = L.a_glu;
     p.a_vec = ((reinterpret_cast<uintptr_t>(L.A) & 15) == 0 && L.lda % 4 == 0 && L.a_zoff % 4 == 0) ? 1 : 0;
     p.b_vec = ((reinterpret_cast<uintptr_t>(L.B) & 15) == 0 && L.ldb % 8 == 0 && L.b_zoff % 8 == 0) ? 1 : 0;
     if (!L.grp_off && L.M <= kGemvMaxRows) {
@@ -325,9 +351,13 @@ int launch_linear(const Linear& L, bool f32, hipStream_t s) {
         ZG_HIP(hipGetLastError());
         return ZG_OK;
     }
+    ZG_REQUIRE(L.a_glu == 0, ZG_ERR_ARG, "linear: the gated activation on load is for steps of few rows");
     ZG_REQUIRE(!(L.z_group && L.grp_off), ZG_ERR_ARG, "linear: a matrix per batch and row groups exclude each other");
     auto tiles = [&](int b) { return (long long)((L.M + b - 1) / b + (L.grp_off ? L.n_groups : 0)) * ((L.N + b - 1) / b) * L.nz; };
-    const bool big = tiles(128) >= 512;
+    // 128 x 128 tiles once they fill the chip twice over; ZGPT2_LM_GEMM_TILE=64|128 pins the choice (tests run small shapes
+    // through the large tiles with it)
+    bool big = tiles(128) >= 512;
+    if (const char* e = getenv("ZGPT2_LM_GEMM_TILE")) big = atoi(e) == 128 ? true : atoi(e) == 64 ? false : big;
     const int b = big ? 128 : 64;
     const dim3 grid((L.N + b - 1) / b, (L.M + b - 1) / b + (L.grp_off ? L.n_groups : 0), L.nz);
     ZG_REQUIRE(grid.y <= 65535 && grid.z <= 65535, ZG_ERR_UNSUPPORTED, "linear: %d rows in %d batches exceed the grid", L.M, L.nz);

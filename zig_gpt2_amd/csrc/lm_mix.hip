@@ -94,6 +94,22 @@ __global__ __launch_bounds__(256) void norm_add_kernel(float* x, const float* y,
     for (int i = threadIdx.x; i < W; i += blockDim.x) x[(size_t)m * W + i] += yr[i] * r * (1.0f + w[i]);
 }
 
+// x += norm(y) * (1 + wb), then h = norm(x) * (1 + wn): the norm behind the mixer, the residual sum and the norm in front of the
+// feed-forward in one pass over the row
+__global__ __launch_bounds__(256) void norm_add_norm_kernel(float* x, const float* y, const float* wb, const float* wn, float eps, float* h, int W) {
+    __shared__ float s_red[8];
+    const int m = blockIdx.x;
+    const float* yr = y + (size_t)m * W;
+    float* xr = x + (size_t)m * W;
+    const float r = row_inv_rms(yr, W, eps, s_red);
+    for (int i = threadIdx.x; i < W; i += blockDim.x) xr[i] += yr[i] * r * (1.0f + wb[i]);  // each thread rereads only what it wrote
+    float ss = 0.0f;
+    for (int i = threadIdx.x; i < W; i += blockDim.x) ss = fmaf(xr[i], xr[i], ss);
+    ss = block_allsum(ss, s_red);
+    const float r2 = 1.0f / sqrtf(ss / (float)W + eps);
+    for (int i = threadIdx.x; i < W; i += blockDim.x) h[(size_t)m * W + i] = xr[i] * r2 * (1.0f + wn[i]);
+}
+
 __global__ __launch_bounds__(256) void norm_gather_kernel(const float* x, const int* rows, const float* w, float eps, float* out, int W) {
     __shared__ float s_red[8];
     const int j = blockIdx.x;
@@ -115,16 +131,6 @@ __global__ __launch_bounds__(256) void norm_plain_kernel(float* v, int ld, int r
 }
 
 // ------------------------------------------------------------------------------------------------ HGRN2
-__global__ __launch_bounds__(256) void hgrn2_gates_kernel(float* proj, int ld, int M, int HD, const float* bias, const float* low) {
-    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= (size_t)M * HD) return;
-    const int m = (int)(idx / HD), i = (int)(idx % HD);
-    float* row = proj + (size_t)m * ld;
-    row[i] = silu_f(row[i]);
-    const float l = low[i];
-    row[HD + i] = l + (1.0f - l) * sigmoid_f(row[HD + i] + bias[i]);
-}
-
 // A column j of a head's state S[D][V] is held by G consecutive lanes, 16 rows each (D <= 16 G).  The token loop is serial; the
 // gates and values of the next SB tokens are staged in the LDS (rows beyond D padded with q = 0, f = 1: they stay zero).
 //
@@ -153,7 +159,7 @@ __device__ __forceinline__ bool scan_find_chunk(int id, const int* ent_len, int 
 template <int G>
 __global__ __launch_bounds__(256) void hgrn2_scan_kernel(const float* proj, int ld, float* out, int ldo, float* state, size_t slot_stride,
                                                          const int* ent_start, const int* ent_len, const int* ent_slot, int n_entries, int H, int D,
-                                                         int V, int mode, int SB, float* wsB, float* wsA) {
+                                                         int V, int mode, int SB, float* wsB, float* wsA, const float* bias, const float* low) {
     extern __shared__ __attribute__((aligned(16))) float s_scan[];
     constexpr int Dp = G * kScanRows;
     const int cols = blockDim.x / G;
@@ -192,8 +198,15 @@ __global__ __launch_bounds__(256) void hgrn2_scan_kernel(const float* proj, int 
         for (int idx = threadIdx.x; idx < nb * Dp; idx += blockDim.x) {
             const int tt = idx / Dp, i = idx % Dp;
             const float* row = proj + (size_t)(m0 + tb + tt) * ld;
-            sq[idx] = i < D ? row[h * D + i] : 0.0f;
-            sf[idx] = i < D ? row[HD + h * D + i] : 1.0f;
+            // the gates are activated on their way into the LDS: q = silu(.), f = low + (1 - low) sigmoid(. + bias)
+            float qv = 0.0f, fv = 1.0f;
+            if (i < D) {
+                const float l = low[h * D + i];
+                qv = silu_f(row[h * D + i]);
+                fv = l + (1.0f - l) * sigmoid_f(row[HD + h * D + i] + bias[h * D + i]);
+            }
+            sq[idx] = qv;
+            sf[idx] = fv;
         }
         for (int idx = threadIdx.x; idx < nb * cols; idx += blockDim.x) {
             const int tt = idx / cols, jj = idx % cols;
@@ -472,31 +485,53 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(const float*
     float mx = -INFINITY, lsum = 0.0f;
     const bool vec = (DT % 4 == 0) && ((reinterpret_cast<uintptr_t>(cache) & 15) == 0);
 
-    for (int kt = 0; kt * 32 < n_keys; ++kt) {
-        __syncthreads();  // the previous tile has been consumed
-        for (int idx = tid; idx < 32 * (DTp / 4); idx += 256) {
+    // a tile's rows travel global -> registers -> LDS; the registers of tile kt + 1 are filled while tile kt is multiplied
+    constexpr int ITEMS = 32 * (DTp / 4) / 256;  // float4 pieces per thread and tile (NKS is even)
+    f32x4 stage[ITEMS];
+    auto fetch = [&](int kt) {
+#pragma unroll
+        for (int it = 0; it < ITEMS; ++it) {
+            const int idx = tid + 256 * it;
             const int key = idx / (DTp / 4), d4 = (idx % (DTp / 4)) * 4, kpos = kt * 32 + key;
-            float v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+            f32x4 x = {0.0f, 0.0f, 0.0f, 0.0f};
             if (kpos < n_keys) {
                 const float* row = cache + ((size_t)pt[kpos / page_tokens] * page_tokens + kpos % page_tokens) * DT;
                 if (vec && d4 + 4 <= DT) {
-                    const f32x4 x = *reinterpret_cast<const f32x4*>(row + d4);
-                    v[0] = x.x; v[1] = x.y; v[2] = x.z; v[3] = x.w;
+                    x = *reinterpret_cast<const f32x4*>(row + d4);
                 } else {
-#pragma unroll
-                    for (int u = 0; u < 4; ++u) v[u] = d4 + u < DT ? row[d4 + u] : 0.0f;
+                    x.x = d4 + 0 < DT ? row[d4 + 0] : 0.0f;
+                    x.y = d4 + 1 < DT ? row[d4 + 1] : 0.0f;
+                    x.z = d4 + 2 < DT ? row[d4 + 2] : 0.0f;
+                    x.w = d4 + 3 < DT ? row[d4 + 3] : 0.0f;
                 }
             }
+            stage[it] = x;
+        }
+    };
+    fetch(0);
+    for (int kt = 0; kt * 32 < n_keys; ++kt) {
+        __syncthreads();  // the previous tile has been consumed
+#pragma unroll
+        for (int it = 0; it < ITEMS; ++it) {
+            const int idx = tid + 256 * it;
+            const int key = idx / (DTp / 4), d4 = (idx % (DTp / 4)) * 4;
             u32x2 pk;
-            pk.x = cvt_pk_bf16(v[0], v[1]);
-            pk.y = cvt_pk_bf16(v[2], v[3]);
+            pk.x = cvt_pk_bf16(stage[it].x, stage[it].y);
+            pk.y = cvt_pk_bf16(stage[it].z, stage[it].w);
             *reinterpret_cast<u32x2*>(&Ks[key * KS_LD + d4]) = pk;
-            if (d4 < NT * 32) {
-                Vt[(d4 + 0) * VT_LD + key] = (bf16_t)(pk.x & 0xFFFFu);
-                Vt[(d4 + 1) * VT_LD + key] = (bf16_t)(pk.x >> 16);
-                Vt[(d4 + 2) * VT_LD + key] = (bf16_t)(pk.y & 0xFFFFu);
-                Vt[(d4 + 3) * VT_LD + key] = (bf16_t)(pk.y >> 16);
-            }
+        }
+        __syncthreads();
+        if ((kt + 1) * 32 < n_keys) fetch(kt + 1);
+        // the latent part once more, transposed: consecutive lanes take consecutive keys, so the 2-byte stores of a wave fall into
+        // consecutive words (written from the rows above rather than beside them: a lane of the loop above holds four dimensions
+        // of ONE key, and its four stores would all hit the same two banks)
+        for (int idx = tid; idx < 32 * (NT * 8); idx += 256) {
+            const int key = idx & 31, d4 = (idx >> 5) * 4;
+            const u32x2 pk = *reinterpret_cast<const u32x2*>(&Ks[key * KS_LD + d4]);
+            Vt[(d4 + 0) * VT_LD + key] = (bf16_t)(pk.x & 0xFFFFu);
+            Vt[(d4 + 1) * VT_LD + key] = (bf16_t)(pk.x >> 16);
+            Vt[(d4 + 2) * VT_LD + key] = (bf16_t)(pk.y & 0xFFFFu);
+            Vt[(d4 + 3) * VT_LD + key] = (bf16_t)(pk.y >> 16);
         }
         __syncthreads();
         if (!head_ok) continue;
@@ -516,25 +551,33 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(const float*
             tmax = fmaxf(tmax, sv[i]);
         }
         tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-        const float mn = fmaxf(mx, tmax);
-        const bool none = mn == -INFINITY;  // a query row beyond the entry: nothing to weigh
-        const float alpha = none ? 1.0f : expf(mx - mn);
+        // The reference point of the exponentials moves only when some query's maximum grew by more than 8 (the weights then
+        // reach e^8 at most, far inside fp32 and bf16 range): the accumulators are rescaled on few tiles instead of on every one.
+        const bool grow = tmax > mx + 8.0f;  // also the first tile of a query (mx = -inf)
         float psum = 0.0f, pv[16];
+        if (__any(grow)) {
+            const float mn = grow ? tmax : mx;
+            const float alpha = (mn == -INFINITY || mx == mn) ? 1.0f : __expf(mx - mn);  // mx = -inf, mn finite: 0
+            lsum *= alpha;
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) o[t][i] *= alpha;
+            mx = mn;
+        }
+        const bool none = mx == -INFINITY;  // a query row beyond the entry: nothing to weigh
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-            pv[i] = none ? 0.0f : expf(sv[i] - mn);
+            pv[i] = none ? 0.0f : __expf(sv[i] - mx);
             psum += pv[i];
         }
-        lsum = lsum * alpha + psum;
-        mx = mn;
+        lsum += psum;
         u32x4 p0, p1;
         p0.x = cvt_pk_bf16(pv[0], pv[1]); p0.y = cvt_pk_bf16(pv[2], pv[3]); p0.z = cvt_pk_bf16(pv[4], pv[5]); p0.w = cvt_pk_bf16(pv[6], pv[7]);
         p1.x = cvt_pk_bf16(pv[8], pv[9]); p1.y = cvt_pk_bf16(pv[10], pv[11]); p1.z = cvt_pk_bf16(pv[12], pv[13]); p1.w = cvt_pk_bf16(pv[14], pv[15]);
         const bf16x8 pf0 = __builtin_bit_cast(bf16x8, p0), pf1 = __builtin_bit_cast(bf16x8, p1);
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
-#pragma unroll
-            for (int i = 0; i < 16; ++i) o[t][i] *= alpha;
             const bf16_t* vrow = &Vt[(t * 32 + r) * VT_LD + 4 * hf];
             const u32x2 a0 = *reinterpret_cast<const u32x2*>(vrow), a1 = *reinterpret_cast<const u32x2*>(vrow + 8);
             const u32x2 b0 = *reinterpret_cast<const u32x2*>(vrow + 16), b1 = *reinterpret_cast<const u32x2*>(vrow + 24);
@@ -555,24 +598,31 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(const float*
         }
 }
 
-// ctx[m][h] from the n_split partials of latent_attention_kernel (fixed order: the result does not depend on timing)
-__global__ __launch_bounds__(256) void latent_merge_kernel(const float* ws, float* ctx, int H, int KR, int n_split) {
-    const int m = blockIdx.x, h = blockIdx.y;
+// ctx[m][h] from the partials of latent_attention_kernel, in a fixed order (the result does not depend on timing); only the
+// ranges that held keys are read
+__global__ __launch_bounds__(256) void latent_merge_kernel(const float* ws, float* ctx, int H, int KR, int n_split, const int* row_pos) {
+    __shared__ float s_w[64];
+    __shared__ float s_L;
+    const int m = blockIdx.x, h = blockIdx.y, n_keys = row_pos[m] + 1;
+    int chunk = (n_keys + n_split - 1) / n_split;
+    chunk = max(64, (chunk + 15) & ~15);
+    const int used = min(n_split, (n_keys + chunk - 1) / chunk);
     const float* part = ws + ((size_t)m * H + h) * n_split * (KR + 2);
-    float M = -INFINITY;
-    for (int sidx = 0; sidx < n_split; ++sidx) M = fmaxf(M, part[(size_t)sidx * (KR + 2)]);
-    float L = 0.0f;
-    for (int sidx = 0; sidx < n_split; ++sidx) {
-        const float pm = part[(size_t)sidx * (KR + 2)];
-        if (pm != -INFINITY) L += expf(pm - M) * part[(size_t)sidx * (KR + 2) + 1];
+    if (threadIdx.x < 64) {
+        const int sidx = threadIdx.x;
+        const float pm = sidx < used ? part[(size_t)sidx * (KR + 2)] : -INFINITY;
+        const float M = wave_allmax(pm);
+        const float w = pm == -INFINITY ? 0.0f : expf(pm - M);
+        s_w[sidx] = w;
+        const float L = wave_allsum(sidx < used ? w * part[(size_t)sidx * (KR + 2) + 1] : 0.0f);
+        if (sidx == 0) s_L = L;
     }
+    __syncthreads();
     float* out = ctx + ((size_t)m * H + h) * KR;
+    const float L = s_L;
     for (int d = threadIdx.x; d < KR; d += blockDim.x) {
         float a = 0.0f;
-        for (int sidx = 0; sidx < n_split; ++sidx) {
-            const float pm = part[(size_t)sidx * (KR + 2)];
-            if (pm != -INFINITY) a = fmaf(expf(pm - M), part[(size_t)sidx * (KR + 2) + 2 + d], a);
-        }
+        for (int sidx = 0; sidx < used; ++sidx) a = fmaf(s_w[sidx], part[(size_t)sidx * (KR + 2) + 2 + d], a);
         out[d] = a / L;
     }
 }
@@ -668,6 +718,13 @@ int launch_norm_add(float* x, const float* y, const float* w, float eps, int M, 
     return ZG_OK;
 }
 
+int launch_norm_add_norm(float* x, const float* y, const float* wb, const float* wn, float eps, float* h, int M, int W, hipStream_t s) {
+    if (M <= 0) return ZG_OK;
+    norm_add_norm_kernel<<<M, 256, 0, s>>>(x, y, wb, wn, eps, h, W);
+    ZG_HIP(hipGetLastError());
+    return ZG_OK;
+}
+
 int launch_norm_gather(const float* x, const int* rows, const float* w, float eps, float* out, int n_rows, int W, hipStream_t s) {
     if (n_rows <= 0) return ZG_OK;
     norm_gather_kernel<<<n_rows, 256, 0, s>>>(x, rows, w, eps, out, W);
@@ -683,17 +740,9 @@ int launch_norm_plain(float* v, int ld, int rows_per_m, int width, int M, const 
     return ZG_OK;
 }
 
-int launch_hgrn2_gates(float* proj, int ld, int M, int HD, const float* bias, const float* low, hipStream_t s) {
-    const size_t n = (size_t)M * HD;
-    if (n == 0) return ZG_OK;
-    hgrn2_gates_kernel<<<(unsigned)((n + 255) / 256), 256, 0, s>>>(proj, ld, M, HD, bias, low);
-    ZG_HIP(hipGetLastError());
-    return ZG_OK;
-}
-
 int launch_hgrn2_scan(const float* proj, int ld, float* out, int ldo, float* state, size_t slot_stride, const int* ent_start,
-                      const int* ent_len, const int* ent_slot, int n_entries, int M, int H, int D, int V, float* ws, size_t ws_floats,
-                      hipStream_t s) {
+                      const int* ent_len, const int* ent_slot, int n_entries, int M, int H, int D, int V, const float* bias, const float* low,
+                      float* ws, size_t ws_floats, hipStream_t s) {
     if (n_entries <= 0) return ZG_OK;
     ZG_REQUIRE(D >= 1 && D <= 16 * kScanRows, ZG_ERR_UNSUPPORTED, "hgrn2: %d key channels per head (at most %d)", D, 16 * kScanRows);
     int G = 1;
@@ -712,7 +761,7 @@ int launch_hgrn2_scan(const float* proj, int ld, float* out, int ldo, float* sta
     float* wsA = chunked ? ws + (size_t)max_chunks * head_floats : nullptr;
 #define ZG_SCAN(G_, grid_x, mode)                                                                                                                 \
     hgrn2_scan_kernel<G_><<<dim3(grid_x, H, (V + cols - 1) / cols), threads, lds, s>>>(proj, ld, out, ldo, state, slot_stride, ent_start, ent_len, \
-                                                                                        ent_slot, n_entries, H, D, V, mode, SB, wsB, wsA)
+                                                                                        ent_slot, n_entries, H, D, V, mode, SB, wsB, wsA, bias, low)
 #define ZG_SCAN_G(grid_x, mode)                    \
     switch (G) {                                   \
         case 1: ZG_SCAN(1, grid_x, mode); break;   \
@@ -803,7 +852,7 @@ int launch_latent_attention(const float* qa, float* ctx, int M, int H, int KR, i
 #undef ZG_ATT
     ZG_HIP(hipGetLastError());
     if (n_split > 1) {
-        latent_merge_kernel<<<dim3(M, H), 256, 0, s>>>(ws, ctx, H, KR, n_split);
+        latent_merge_kernel<<<dim3(M, H), 256, 0, s>>>(ws, ctx, H, KR, n_split, row_pos);
         ZG_HIP(hipGetLastError());
     }
     return ZG_OK;

@@ -31,6 +31,7 @@
 #include <string>
 #include <vector>
 
+#include "lm_host.hpp"
 #include "../../include/zgpt2_ops.hpp"
 
 using ops::Slice;
@@ -432,8 +433,9 @@ static int main_multi_gpu(int world, bool plan_only, const GPTConfig& c, const s
 }
 
 int main(int argc, char** argv) {
+    if (argc >= 2 && std::string(argv[1]) == "lm") return lmhost::lm_main(argc, argv);  // a checkpoint folder of the layered-model tier
     if (argc < 5) {
-        fprintf(stderr, "usage: %s <tiny|tiny3|nano-char|124M> <seed | raw weight dir> <tok,tok,...> <n_steps> [--model-tier]\n", argv[0]);
+        fprintf(stderr, "usage: %s <tiny|tiny3|nano-char|124M> <seed | raw weight dir> <tok,tok,...> <n_steps> [--model-tier]\n       %s lm <checkpoint dir> <tok,tok,...[;tok,...]> <n_new> [--dtype bfloat16|float32] [--temp T] [--seed S]\n", argv[0], argv[0]);
         return 2;
     }
     const std::string name = argv[1];
