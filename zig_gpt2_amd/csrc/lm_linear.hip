@@ -95,18 +95,19 @@ __global__ __launch_bounds__(256) void lm_gemv_kernel(const LinArgs p) {
     for (int m = 0; m < MR; ++m) acc0[m] = acc1[m] = 0.0f;
     // two K pieces per trip, all four weight vectors requested before the first is used: rows of up to 1024 columns cost one
     // memory round trip
-    for (int k = lane * 8; k < p.K; k += 1024) {
-        float wa[2][8], wb[2][8];
+    constexpr int U = MR <= 2 ? 2 : 1;
+    for (int k = lane * 8; k < p.K; k += 512 * U) {
+        float wa[U][8], wb[U][8];
 #pragma unroll
-        for (int u = 0; u < 2; ++u) {
+        for (int u = 0; u < U; ++u) {
             load_w8(w0, k + 512 * u, p.K, p.b_vec, wa[u]);
             load_w8(w1, k + 512 * u, p.K, p.b_vec, wb[u]);
         }
 #pragma unroll
         for (int m = 0; m < MR; ++m) {
-            f32x4 av[2][2];
+            f32x4 av[U][2];
 #pragma unroll
-            for (int u = 0; u < 2; ++u) {
+            for (int u = 0; u < U; ++u) {
                 const int kk = k + 512 * u;
                 f32x4 a0 = load_a4(arow[m], kk, p.K, p.a_vec), a1 = load_a4(arow[m], kk + 4, p.K, p.a_vec);
                 if (p.a_glu > 0 && arow[m]) {  // rows [gate | up]: silu(gate) * up
@@ -122,7 +123,7 @@ __global__ __launch_bounds__(256) void lm_gemv_kernel(const LinArgs p) {
             }
             float s0 = acc0[m], s1 = acc1[m];
 #pragma unroll
-            for (int u = 0; u < 2; ++u) {
+            for (int u = 0; u < U; ++u) {
                 const f32x4 a0 = av[u][0], a1 = av[u][1];
                 s0 = fmaf(a0.x, wa[u][0], s0); s1 = fmaf(a0.x, wb[u][0], s1);
                 s0 = fmaf(a0.y, wa[u][1], s0); s1 = fmaf(a0.y, wb[u][1], s1);
