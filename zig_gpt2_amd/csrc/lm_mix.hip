@@ -43,14 +43,58 @@ __global__ __launch_bounds__(256) void embed_kernel(const bf16_t* table, const i
     for (int i = threadIdx.x; i < W; i += blockDim.x) x[(size_t)m * W + i] = ok ? __uint_as_float((uint32_t)row[i] << 16) : 0.0f;
 }
 
+// Rows of up to 256 * kRowRegs floats are held in registers between the statistics and the result: every operand is requested
+// in one go at the top of the kernel, so a one-row step (decoding) pays one memory round trip instead of one per pass.
+constexpr int kRowRegs = 16;
+
 __global__ __launch_bounds__(256) void norm_shift_kernel(const float* x, const float* w, const float* mu, float eps, float* out, int W,
                                                          const int* row_prev, const int* row_slot, const float* shift_state,
                                                          size_t slot_stride, const int* row_entry_if_last, float* last_out) {
     __shared__ float s_red[8];
     const int m = blockIdx.x;
     const float* xr = x + (size_t)m * W;
-    const float r = row_inv_rms(xr, W, eps, s_red);
     const int entry = row_entry_if_last ? row_entry_if_last[m] : -1;
+    const int pm = mu ? row_prev[m] : -1;
+    const float* xp = (mu && pm >= 0) ? x + (size_t)pm * W : nullptr;
+    const float* hp = (mu && pm < 0) ? shift_state + (size_t)row_slot[m] * slot_stride : nullptr;
+    if (W <= 256 * kRowRegs) {
+        float xv[kRowRegs], pv[kRowRegs], wv[kRowRegs], mv[kRowRegs];
+#pragma unroll
+        for (int j = 0; j < kRowRegs; ++j) {
+            const int i = threadIdx.x + 256 * j;
+            const bool ok = i < W;
+            xv[j] = ok ? xr[i] : 0.0f;
+            wv[j] = ok ? w[i] : 0.0f;
+            mv[j] = (ok && mu) ? mu[i] : 0.0f;
+            pv[j] = !ok ? 0.0f : xp ? xp[i] : hp ? hp[i] : 0.0f;
+        }
+        float ss = 0.0f;  // the same order as row_inv_rms: element i of thread t is t + 256 j, j ascending
+#pragma unroll
+        for (int j = 0; j < kRowRegs; ++j) ss = fmaf(xv[j], xv[j], ss);
+        ss = block_allsum(ss, s_red);
+        const float r = 1.0f / sqrtf(ss / (float)W + eps);
+        float rp = 0.0f;
+        if (xp) {
+            float sp = 0.0f;
+#pragma unroll
+            for (int j = 0; j < kRowRegs; ++j) sp = fmaf(pv[j], pv[j], sp);
+            sp = block_allsum(sp, s_red);
+            rp = 1.0f / sqrtf(sp / (float)W + eps);
+        }
+#pragma unroll
+        for (int j = 0; j < kRowRegs; ++j) {
+            const int i = threadIdx.x + 256 * j;
+            if (i < W) {
+                const float g = 1.0f + wv[j];
+                const float h = xv[j] * r * g;
+                const float before = xp ? pv[j] * rp * g : pv[j];
+                out[(size_t)m * W + i] = mu ? h + (before - h) * mv[j] : h;
+                if (entry >= 0) last_out[(size_t)entry * W + i] = h;
+            }
+        }
+        return;
+    }
+    const float r = row_inv_rms(xr, W, eps, s_red);
     if (mu == nullptr) {
         for (int i = threadIdx.x; i < W; i += blockDim.x) {
             const float h = xr[i] * r * (1.0f + w[i]);
@@ -59,16 +103,8 @@ __global__ __launch_bounds__(256) void norm_shift_kernel(const float* x, const f
         }
         return;
     }
-    const int pm = row_prev[m];
-    const float* xp = nullptr;
-    const float* hp = nullptr;
     float rp = 0.0f;
-    if (pm >= 0) {
-        xp = x + (size_t)pm * W;
-        rp = row_inv_rms(xp, W, eps, s_red);
-    } else {
-        hp = shift_state + (size_t)row_slot[m] * slot_stride;
-    }
+    if (xp) rp = row_inv_rms(xp, W, eps, s_red);
     for (int i = threadIdx.x; i < W; i += blockDim.x) {
         const float g = 1.0f + w[i];
         const float h = xr[i] * r * g;
@@ -101,6 +137,40 @@ __global__ __launch_bounds__(256) void norm_add_norm_kernel(float* x, const floa
     const int m = blockIdx.x;
     const float* yr = y + (size_t)m * W;
     float* xr = x + (size_t)m * W;
+    if (W <= 256 * kRowRegs) {
+        float yv[kRowRegs], xv[kRowRegs], bv[kRowRegs], nv[kRowRegs];
+#pragma unroll
+        for (int j = 0; j < kRowRegs; ++j) {
+            const int i = threadIdx.x + 256 * j;
+            const bool ok = i < W;
+            yv[j] = ok ? yr[i] : 0.0f;
+            xv[j] = ok ? xr[i] : 0.0f;
+            bv[j] = ok ? wb[i] : 0.0f;
+            nv[j] = ok ? wn[i] : 0.0f;
+        }
+        float ss = 0.0f;
+#pragma unroll
+        for (int j = 0; j < kRowRegs; ++j) ss = fmaf(yv[j], yv[j], ss);
+        ss = block_allsum(ss, s_red);
+        const float r = 1.0f / sqrtf(ss / (float)W + eps);
+        float s2 = 0.0f;
+#pragma unroll
+        for (int j = 0; j < kRowRegs; ++j) {
+            xv[j] += yv[j] * r * (1.0f + bv[j]);  // (rows beyond W: 0 + 0)
+            s2 = fmaf(xv[j], xv[j], s2);
+        }
+        s2 = block_allsum(s2, s_red);
+        const float r2 = 1.0f / sqrtf(s2 / (float)W + eps);
+#pragma unroll
+        for (int j = 0; j < kRowRegs; ++j) {
+            const int i = threadIdx.x + 256 * j;
+            if (i < W) {
+                xr[i] = xv[j];
+                h[(size_t)m * W + i] = xv[j] * r2 * (1.0f + nv[j]);
+            }
+        }
+        return;
+    }
     const float r = row_inv_rms(yr, W, eps, s_red);
     for (int i = threadIdx.x; i < W; i += blockDim.x) xr[i] += yr[i] * r * (1.0f + wb[i]);  // each thread rereads only what it wrote
     float ss = 0.0f;

@@ -23,39 +23,53 @@ __device__ __forceinline__ float block_allsum(float v, float* s_red) {
     return t;
 }
 
-// one wave per row: the lanes split the row's W channels (four at a time), a router row is one dot product summed over the
-// wave; lane e % 64 keeps the logit of expert e (experts e, e + 64, e + 128, e + 192 in its four slots)
+// One workgroup per row.  The four waves share the experts (wave w scores experts w, w + 4, ...): a router row is one dot
+// product, the lanes take 16-byte pieces of it and every piece of up to 2048 channels is requested before the first is used; the
+// logits meet in the LDS and wave 0 does the softmax and the choice, lane e % 64 holding expert e (four slots per lane).
 __global__ __launch_bounds__(256) void route_kernel(const float* g, int M, int W, const bf16_t* router, const float* correction, int E, int top,
                                                     int* pick, float* weight) {
-    const int m = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
-    if (m >= M) return;
+    __shared__ float s_z[kMaxExperts];
+    const int m = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const float* row = g + (size_t)m * W;
-    float z[4], sc[4], ch[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) z[i] = -INFINITY;
-    const bool vec = (W % 4 == 0) && ((reinterpret_cast<uintptr_t>(g) & 15) == 0) && ((reinterpret_cast<uintptr_t>(router) & 7) == 0);
-    for (int e = 0; e < E; ++e) {
+    const bool vec = (W % 8 == 0) && ((reinterpret_cast<uintptr_t>(g) & 15) == 0) && ((reinterpret_cast<uintptr_t>(router) & 15) == 0);
+    for (int e = wave; e < E; e += 4) {
         const bf16_t* wr = router + (size_t)e * W;
         float a = 0.0f;
         if (vec) {
-            for (int k = lane * 4; k < W; k += 256) {
-                const f32x4 x = *reinterpret_cast<const f32x4*>(row + k);
-                const u32x2 w2 = *reinterpret_cast<const u32x2*>(wr + k);
-                a = fmaf(x.x, bf16_lo(w2.x), a);
-                a = fmaf(x.y, bf16_hi(w2.x), a);
-                a = fmaf(x.z, bf16_lo(w2.y), a);
-                a = fmaf(x.w, bf16_hi(w2.y), a);
+            for (int k0 = lane * 8; k0 < W; k0 += 2048) {
+                f32x4 x0[4], x1[4];
+                u32x4 wv[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const int k = k0 + 512 * u;
+                    const bool ok = k < W;
+                    x0[u] = ok ? *reinterpret_cast<const f32x4*>(row + k) : f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+                    x1[u] = ok ? *reinterpret_cast<const f32x4*>(row + k + 4) : f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+                    wv[u] = ok ? *reinterpret_cast<const u32x4*>(wr + k) : u32x4{0u, 0u, 0u, 0u};
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    a = fmaf(x0[u].x, bf16_lo(wv[u].x), a);
+                    a = fmaf(x0[u].y, bf16_hi(wv[u].x), a);
+                    a = fmaf(x0[u].z, bf16_lo(wv[u].y), a);
+                    a = fmaf(x0[u].w, bf16_hi(wv[u].y), a);
+                    a = fmaf(x1[u].x, bf16_lo(wv[u].z), a);
+                    a = fmaf(x1[u].y, bf16_hi(wv[u].z), a);
+                    a = fmaf(x1[u].z, bf16_lo(wv[u].w), a);
+                    a = fmaf(x1[u].w, bf16_hi(wv[u].w), a);
+                }
             }
         } else {
             for (int k = lane; k < W; k += 64) a = fmaf(row[k], __uint_as_float((uint32_t)wr[k] << 16), a);
         }
         a = wave_allsum(a);
-        if ((e & 63) == lane) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-                if ((e >> 6) == i) z[i] = a;
-        }
+        if (lane == 0) s_z[e] = a;
     }
+    __syncthreads();
+    if (wave != 0) return;
+    float z[4], sc[4], ch[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) z[i] = lane + 64 * i < E ? s_z[lane + 64 * i] : -INFINITY;
     const float mx = wave_allmax(fmaxf(fmaxf(z[0], z[1]), fmaxf(z[2], z[3])));
     float sum = 0.0f;
 #pragma unroll
@@ -160,7 +174,7 @@ int launch_route(const float* g, int M, int W, const bf16_t* router, const float
     if (M <= 0) return ZG_OK;
     ZG_REQUIRE(E >= 1 && E <= kMaxExperts && top >= 1 && top <= E, ZG_ERR_UNSUPPORTED, "router: %d experts, %d chosen (at most %d experts)", E, top,
                kMaxExperts);
-    route_kernel<<<(M + 3) / 4, 256, 0, s>>>(g, M, W, router, correction, E, top, pick, weight);
+    route_kernel<<<M, 256, 0, s>>>(g, M, W, router, correction, E, top, pick, weight);
     ZG_HIP(hipGetLastError());
     return ZG_OK;
 }
