@@ -386,3 +386,24 @@ def test_checkpoint_folder_through_registry_host_program_and_trace_replay(tmp_pa
     tl.assert_close(rd(3), ref[9:10], "float32")
     tl.assert_close(rd(4), ref[10:11], "float32")
     tl.assert_close(rd(5), ref[10:11], "float32")
+
+
+def test_scheduler_serves_more_requests_than_slots():
+    """Continuous batching: seven requests of unequal lengths on two slots and a cache that holds about two of them — every
+    request's tokens equal its generation alone, slots and pages go round."""
+    cfg = full_cfg(loop={"start": 0, "stop": 2, "times": 2})
+    w = tl.weights(cfg, seed=18, head_std=1.0)
+    m = make(cfg, w, max_tokens=128, max_seqs=2, page_tokens=8)
+    reqs = [(tl.tokens(90 + i, n, cfg["vocab"]), k) for i, (n, k) in enumerate([(30, 6), (3, 9), (17, 2), (1, 12), (41, 5), (8, 8), (2, 1)])]
+    alone = [m.generate([p], k)[0] for p, k in reqs]
+    total = m.free_tokens()
+    sch = lm.Scheduler(m, portion=16)
+    ids = [sch.submit(p, k) for p, k in reqs]
+    out = sch.run()
+    for rid, want in zip(ids, alone):
+        assert np.array_equal(out[rid], want), (rid, out[rid], want)
+    assert m.free_tokens() == total and sch._reserved == 0
+    assert sch.steps < sum(-(-len(p) // 16) + k for p, k in reqs)  # requests shared steps
+    with pytest.raises(Exception):
+        lm.Scheduler(m).submit([], 3)
+    m.close()

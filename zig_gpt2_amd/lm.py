@@ -169,6 +169,7 @@ class LayeredLM:
         check(L.zg_lm_create(C.byref(h), C.byref(cfg), device))
         self.h = h
         self.n_passes = len(config.passes())
+        self.page_tokens = int(page_tokens) or 64  # (the library's default)
 
     @classmethod
     def from_dir(cls, path, dtype="bfloat16", **kw):
@@ -285,3 +286,81 @@ class LayeredLM:
         buf = C.create_string_buffer(160)
         self._L.zg_debug_last_kernel(buf, len(buf))
         return buf.value.decode()
+
+
+class Scheduler:
+    """Continuous batching over one LayeredLM.  Requests wait in a queue and are admitted while a state slot and enough cache
+    pages for their whole life (prompt + new tokens) are free; every iteration is ONE ragged step of the library: the next
+    portion (at most `portion` tokens) of every prompt that is still being fed, beside the single last token of every sequence
+    that is decoding.  A finished request gives its slot and pages back at once, and the next one in the queue takes them.
+    Token choice: greedy (temp == 0, first maximum) or softmax(logits / temp) sampling from a generator seeded per request."""
+
+    def __init__(self, model: LayeredLM, portion=256, temp=0.0, seed=0):
+        self.model, self.portion, self.temp, self.seed, self.page = model, int(portion), float(temp), int(seed), model.page_tokens
+        self.queue, self.active, self.done, self._next_id, self._reserved = [], [], {}, 0, 0
+        self.steps = 0
+
+    def submit(self, prompt, n_new):
+        rid = self._next_id
+        self._next_id += 1
+        prompt = np.ascontiguousarray(prompt, dtype=np.int32).reshape(-1)
+        if prompt.size < 1 or n_new < 1:
+            raise ValueError("a request needs a prompt and at least one new token")
+        self.queue.append({"id": rid, "prompt": prompt, "n_new": int(n_new), "fed": 0, "out": [], "seq": None,
+                           "rng": np.random.default_rng([self.seed, rid])})
+        return rid
+
+    def _pages(self, r):
+        return -(-(r["prompt"].size + r["n_new"]) // self.page) * self.page
+
+    def _admit(self):
+        while self.queue:
+            r = self.queue[0]
+            if self.model.free_tokens() - self._reserved < self._pages(r):
+                break
+            try:
+                r["seq"] = self.model.open()
+            except _lib.ZgError:
+                break  # no slot
+            self._reserved += self._pages(r)
+            self.active.append(self.queue.pop(0))
+
+    def _choose(self, r, logits):
+        if self.temp <= 0.0:
+            return int(np.argmax(logits))
+        z = logits.astype(np.float64) / self.temp
+        p = np.exp(z - z.max())
+        return int(r["rng"].choice(p.size, p=p / p.sum()))
+
+    def run(self):
+        """Serve every submitted request; returns {request id: new tokens}."""
+        while self.queue or self.active:
+            self._admit()
+            if not self.active:
+                raise RuntimeError("a request does not fit the cache even when it is alone")
+            entries, asked = [], []
+            for r in self.active:
+                n = r["prompt"].size
+                if r["fed"] < n:  # still feeding the prompt
+                    hi = min(n, r["fed"] + self.portion)
+                    last = hi == n
+                    entries.append((r["seq"], r["prompt"][r["fed"]:hi], [hi - r["fed"] - 1] if last else []))
+                    r["fed"] = hi
+                    if last:
+                        asked.append(r)
+                else:
+                    entries.append((r["seq"], [r["out"][-1]], [0]))
+                    asked.append(r)
+            before = self.model.free_tokens()
+            logits = self.model.step(entries)
+            self._reserved -= before - self.model.free_tokens()  # pages the step took are no longer merely promised
+            self.steps += 1
+            for r, row in zip(asked, logits):
+                r["out"].append(self._choose(r, row))
+            for r in [r for r in self.active if len(r["out"]) >= r["n_new"]]:
+                held = -(-self.model.seq_len(r["seq"]) // self.page) * self.page
+                self._reserved -= self._pages(r) - held  # what was promised and never taken
+                self.model.close_seq(r["seq"])
+                self.active.remove(r)
+                self.done[r["id"]] = np.array(r["out"][: r["n_new"]], np.int32)
+        return self.done
