@@ -375,7 +375,7 @@ int check_layer(const zg_lm_layer& d, size_t i) {
 // The kernels of one portion, from the embedding to the commit of the token-shift rows: launches only, every per-step value
 // (tokens, positions, slots, page tables) is read from device memory — so for a given number of rows and entries the sequence
 // is the same every step and can be replayed from a captured graph (decode steps: one row per entry).
-int enqueue_layers(zg_lm* g, int M, int n_ent, bool capturing) {
+int enqueue_layers(zg_lm* g, int M, int n_ent, bool capturing, bool single) {
     hipStream_t s = g->stream;
     const int W = g->W, MS = g->MS, NS = g->NS;
     const int *d_ids = g->meta, *d_pos = d_ids + MS, *d_slot = d_pos + MS, *d_prev = d_slot + MS, *d_last = d_prev + MS, *d_want = d_last + MS;
@@ -384,13 +384,23 @@ int enqueue_layers(zg_lm* g, int M, int n_ent, bool capturing) {
     const float eps = g->cfg.norm_eps;
     const bool few = M <= kGemvMaxRows;
     ZG_TRY(launch_embed(g->embed, d_ids, g->x, M, W, g->V, g->flag, s));
+    bool h_ready = false;  // g->h already holds this pass's shifted norm (written by the previous pass's fused tail)
     for (int p = 0; p < g->n_passes; ++p) {
         const Pass& ps = g->passes[p];
         const LayerW& L = g->layers[ps.layer];
         const zg_lm_layer& d = L.d;
         const int H = d.heads, D = d.dim, Vd = d.vdim;
-        ZG_TRY(launch_norm_shift(g->x, L.norm1, L.shift, eps, g->h, M, W, d_prev, d_slot, g->shift_state + (size_t)p * W, (size_t)g->n_passes * W,
-                                 d_last, g->last_h + (size_t)p * NS * W, s));
+        if (!h_ready)
+            ZG_TRY(launch_norm_shift(g->x, L.norm1, L.shift, eps, g->h, M, W, d_prev, d_slot, g->shift_state + (size_t)p * W,
+                                     (size_t)g->n_passes * W, d_last, g->last_h + (size_t)p * NS * W, s));
+        h_ready = false;
+        // one row per entry: the pass's last sum is fused with the next pass's norm + shift (tail below)
+        auto tail = [&](const float* y, const float* yexp, const float* weight, int top, const float* wb) -> int {
+            if (!single || p + 1 >= g->n_passes) return ZG_OK;
+            const LayerW& N = g->layers[g->passes[p + 1].layer];
+            return launch_sum_norm_shift(g->x, y, yexp, weight, top, wb, N.norm1, N.shift, eps, g->h, M, W, d_slot, g->shift_state + (size_t)(p + 1) * W,
+                                         (size_t)g->n_passes * W, d_last, g->last_h + (size_t)(p + 1) * NS * W, s, &h_ready);
+        };
         Linear lin;
         if (d.mixer == ZG_LM_MIX_HGRN2) {
             const int HD = H * D, HV = H * Vd, NP = 2 * HD + HV;
@@ -435,7 +445,10 @@ int enqueue_layers(zg_lm* g, int M, int n_ent, bool capturing) {
             ZG_TRY(launch_linear(lin, f32, s));
         }
         if (d.ff != ZG_LM_FF_NONE) ZG_TRY(launch_norm_add_norm(g->x, g->y, L.norm1b, L.norm2, eps, g->h, M, W, s));
-        else ZG_TRY(launch_norm_add(g->x, g->y, L.norm1b, eps, M, W, s));
+        else {
+            ZG_TRY(tail(g->y, nullptr, nullptr, 0, L.norm1b));
+            if (!h_ready) ZG_TRY(launch_norm_add(g->x, g->y, L.norm1b, eps, M, W, s));
+        }
         const int F = d.ff_width;
         if (d.ff == ZG_LM_FF_DENSE) {
             lin = Linear();
@@ -444,7 +457,8 @@ int enqueue_layers(zg_lm* g, int M, int n_ent, bool capturing) {
             lin = Linear();
             lin.A = g->u; lin.lda = F; lin.B = L.down; lin.ldb = F; lin.C = g->y; lin.ldc = W; lin.M = M; lin.N = W; lin.K = F;
             ZG_TRY(launch_linear(lin, f32, s));
-            ZG_TRY(launch_norm_add(g->x, g->y, L.norm2b, eps, M, W, s));
+            ZG_TRY(tail(g->y, nullptr, nullptr, 0, L.norm2b));
+            if (!h_ready) ZG_TRY(launch_norm_add(g->x, g->y, L.norm2b, eps, M, W, s));
         } else if (d.ff == ZG_LM_FF_MOE) {
             const int E = d.experts, top = d.top, NA = M * top;
             ZG_TRY(launch_route(g->h, M, W, L.router, L.correction, E, top, g->pick, g->wt, s));
@@ -466,7 +480,8 @@ int enqueue_layers(zg_lm* g, int M, int n_ent, bool capturing) {
                 ZG_TRY(launch_glu(g->gu_buf, g->hb, NA, F, s));
             }
             ZG_TRY(launch_linear(dn, f32, s));
-            ZG_TRY(launch_moe_combine(g->x, g->ye, few ? nullptr : g->inv, g->wt, top, L.norm2b, eps, M, W, s));
+            if (few) ZG_TRY(tail(nullptr, g->ye, g->wt, top, L.norm2b));
+            if (!h_ready) ZG_TRY(launch_moe_combine(g->x, g->ye, few ? nullptr : g->inv, g->wt, top, L.norm2b, eps, M, W, s));
         }
         if (g->trace && !capturing && (size_t)(p + 1) * M * W <= g->trace_floats) {
             ZG_HIP(hipMemcpyAsync(g->trace + (size_t)p * M * W, g->x, (size_t)M * W * sizeof(float), hipMemcpyDeviceToHost, s));
@@ -519,7 +534,7 @@ int run_portion(zg_lm* g, const std::vector<Piece>& pieces, float* logits_out, c
         if (!g->decode_graph[M]) {
             hipGraph_t graph = nullptr;
             ZG_HIP(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal));
-            const int st = enqueue_layers(g, M, n_ent, true);
+            const int st = enqueue_layers(g, M, n_ent, true, true);
             const hipError_t ce = hipStreamEndCapture(s, &graph);
             if (st != ZG_OK) {
                 if (graph) (void)hipGraphDestroy(graph);
@@ -531,7 +546,9 @@ int run_portion(zg_lm* g, const std::vector<Piece>& pieces, float* logits_out, c
         }
         ZG_HIP(hipGraphLaunch(g->decode_graph[M], s));
     } else {
-        ZG_TRY(enqueue_layers(g, M, n_ent, false));
+        bool one_row = M <= kGemvMaxRows;
+        for (const Piece& pc : pieces) one_row = one_row && pc.n == 1;
+        ZG_TRY(enqueue_layers(g, M, n_ent, false, one_row));
     }
 
     // logits of the rows that were asked for, logit_rows at a time

@@ -64,6 +64,11 @@ int launch_commit_rows(float* dst, size_t slot_stride, const float* src, size_t 
 int launch_norm_add(float* x, const float* y, const float* w, float eps, int M, int W, hipStream_t s);
 // x[m] += y[m] / rms(y[m]) * (1 + wb);  h[m] = x[m] / rms(x[m]) * (1 + wn)   (the two above in one launch)
 int launch_norm_add_norm(float* x, const float* y, const float* wb, const float* wn, float eps, float* h, int M, int W, hipStream_t s);
+// Steps of one row per entry: the sum behind a pass's last sublayer (y, or the weighted sum of the chosen experts' rows yexp) and
+// the next pass's norm + shift in one launch.  *taken = false for rows too wide for its registers (nothing launched).
+int launch_sum_norm_shift(float* x, const float* y, const float* yexp, const float* weight, int top, const float* wb, const float* wn, const float* mu,
+                          float eps, float* out, int M, int W, const int* row_slot, const float* shift_state, size_t slot_stride,
+                          const int* row_entry_if_last, float* last_out, hipStream_t s, bool* taken);
 // out[j] = x[rows[j]] / rms * (1 + w)            (the model's last norm on the rows whose logits are asked for)
 int launch_norm_gather(const float* x, const int* rows, const float* w, float eps, float* out, int n_rows, int W, hipStream_t s);
 // In place over `rows` rows of `width` floats with row stride ld: v / rms(v) * w  (a plain weight; per-head norms)

@@ -180,6 +180,65 @@ __global__ __launch_bounds__(256) void norm_add_norm_kernel(float* x, const floa
     for (int i = threadIdx.x; i < W; i += blockDim.x) h[(size_t)m * W + i] = xr[i] * r2 * (1.0f + wn[i]);
 }
 
+// Steps of one row per entry (decoding): the sum behind a pass's last sublayer and the NEXT pass's norm + token shift in one
+// launch, the row held in registers:
+//   y = a sublayer's output row, or sum_k weight[k] * yexp[m top + k] (the chosen experts, in choice order)
+//   x += norm(y) (1 + wb);   h = norm(x) (1 + wn);   out = h + (state[slot] - h) mu;   last_out[entry] = h
+// (the predecessor of a decoded token is always the row its slot keeps)
+__global__ __launch_bounds__(256) void sum_norm_shift_kernel(float* x, const float* y, const float* yexp, const float* weight, int top, const float* wb,
+                                                             const float* wn, const float* mu, float eps, float* out, int W, const int* row_slot,
+                                                             const float* shift_state, size_t slot_stride, const int* row_entry_if_last,
+                                                             float* last_out) {
+    __shared__ float s_red[8];
+    const int m = blockIdx.x;
+    float* xr = x + (size_t)m * W;
+    const float* hp = shift_state + (size_t)row_slot[m] * slot_stride;
+    const int entry = row_entry_if_last[m];
+    float yv[kRowRegs], xv[kRowRegs], bv[kRowRegs], nv[kRowRegs], mv[kRowRegs], pv[kRowRegs];
+#pragma unroll
+    for (int j = 0; j < kRowRegs; ++j) {
+        const int i = threadIdx.x + 256 * j;
+        const bool ok = i < W;
+        float v = 0.0f;
+        if (ok) {
+            if (yexp) {
+                for (int k = 0; k < top; ++k) v = fmaf(weight[m * top + k], yexp[(size_t)(m * top + k) * W + i], v);
+            } else {
+                v = y[(size_t)m * W + i];
+            }
+        }
+        yv[j] = v;
+        xv[j] = ok ? xr[i] : 0.0f;
+        bv[j] = ok ? wb[i] : 0.0f;
+        nv[j] = ok ? wn[i] : 0.0f;
+        mv[j] = ok ? mu[i] : 0.0f;
+        pv[j] = ok ? hp[i] : 0.0f;
+    }
+    float ss = 0.0f;
+#pragma unroll
+    for (int j = 0; j < kRowRegs; ++j) ss = fmaf(yv[j], yv[j], ss);
+    ss = block_allsum(ss, s_red);
+    const float r = 1.0f / sqrtf(ss / (float)W + eps);
+    float s2 = 0.0f;
+#pragma unroll
+    for (int j = 0; j < kRowRegs; ++j) {
+        xv[j] += yv[j] * r * (1.0f + bv[j]);
+        s2 = fmaf(xv[j], xv[j], s2);
+    }
+    s2 = block_allsum(s2, s_red);
+    const float r2 = 1.0f / sqrtf(s2 / (float)W + eps);
+#pragma unroll
+    for (int j = 0; j < kRowRegs; ++j) {
+        const int i = threadIdx.x + 256 * j;
+        if (i < W) {
+            const float h = xv[j] * r2 * (1.0f + nv[j]);
+            xr[i] = xv[j];
+            out[(size_t)m * W + i] = h + (pv[j] - h) * mv[j];
+            if (entry >= 0) last_out[(size_t)entry * W + i] = h;
+        }
+    }
+}
+
 __global__ __launch_bounds__(256) void norm_gather_kernel(const float* x, const int* rows, const float* w, float eps, float* out, int W) {
     __shared__ float s_red[8];
     const int j = blockIdx.x;
@@ -792,6 +851,18 @@ int launch_norm_add_norm(float* x, const float* y, const float* wb, const float*
     if (M <= 0) return ZG_OK;
     norm_add_norm_kernel<<<M, 256, 0, s>>>(x, y, wb, wn, eps, h, W);
     ZG_HIP(hipGetLastError());
+    return ZG_OK;
+}
+
+int launch_sum_norm_shift(float* x, const float* y, const float* yexp, const float* weight, int top, const float* wb, const float* wn, const float* mu,
+                          float eps, float* out, int M, int W, const int* row_slot, const float* shift_state, size_t slot_stride,
+                          const int* row_entry_if_last, float* last_out, hipStream_t s, bool* taken) {
+    *taken = false;
+    if (M <= 0 || W > 256 * kRowRegs) return ZG_OK;  // wider rows: the caller's separate launches
+    sum_norm_shift_kernel<<<M, 256, 0, s>>>(x, y, yexp, weight, top, wb, wn, mu, eps, out, W, row_slot, shift_state, slot_stride, row_entry_if_last,
+                                            last_out);
+    ZG_HIP(hipGetLastError());
+    *taken = true;
     return ZG_OK;
 }
 
