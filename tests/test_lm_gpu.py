@@ -269,6 +269,27 @@ def test_large_tiles_on_small_shapes(monkeypatch):
         m.close()
 
 
+def test_long_rows_in_decode_steps():
+    """Feed-forward widths beyond 1024: decode steps multiply their down-projections with K split over the waves of a workgroup
+    (one width a multiple of the 16-byte pieces, one not) alone and as a batch of two; a batch of three takes the general kernel."""
+    cfg = tl.config([tl.hgrn2_layer(mlp=tl.dense_mlp(ff=1100)), tl.latent_layer(mlp=tl.dense_mlp(ff=1032))])
+    w = tl.weights(cfg, seed=19)
+    oracle = lm_oracle.Model(cfg, w)
+    toks = [tl.tokens(63 + i, 14, cfg["vocab"]) for i in range(3)]
+    refs = [oracle.forward(t)[0] for t in toks]
+    for dtype in ("float32", "bfloat16"):
+        m = make(cfg, w, dtype)
+        tl.assert_close(run_cut(m, toks[0], range(1, 14)), refs[0], dtype, dtype)
+        for nb in (2, 3):
+            seqs = [m.open() for _ in range(nb)]
+            rows = [m.step([(s, [t[i]], [0]) for s, t in zip(seqs, toks)]) for i in range(14)]
+            for b in range(nb):
+                tl.assert_close(np.stack([r[b] for r in rows]), refs[b], dtype, (dtype, nb, b))
+            for s in seqs:
+                m.close_seq(s)
+        m.close()
+
+
 def test_greedy_and_sampled_generation():
     cfg = full_cfg(loop={"start": 1, "stop": 3, "times": 2})
     w = tl.weights(cfg, seed=14, head_std=1.0)

@@ -148,6 +148,87 @@ __global__ __launch_bounds__(256) void lm_gemv_kernel(const LinArgs p) {
     }
 }
 
+// The same for long rows (K >= 1024): a workgroup owns two weight rows and its four waves split K into quarters, so a matrix of
+// a few MB is requested whole in one go by thousands of waves instead of trip by trip by a few hundred (a 1600 x 1600 matrix:
+// 800 workgroups, every 16-byte piece in flight at once); the quarter sums meet in the LDS.  The summation order of an output
+// depends on K alone.
+template <int MR>
+__global__ __launch_bounds__(256) void lm_gemv_ks_kernel(const LinArgs p) {
+    __shared__ float s_part[4][MR][2];
+    const int z = blockIdx.z, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int n0 = blockIdx.x * 2;
+    const bf16_t* B = p.B + (long long)(p.z_group ? p.z_group[z] : z) * p.b_zoff;
+    const float* A = p.A + (long long)z * p.a_zoff;
+    float* C = p.C + (long long)z * p.c_zoff;
+    const float* arow[MR];
+#pragma unroll
+    for (int m = 0; m < MR; ++m) {
+        arow[m] = nullptr;
+        if (m < p.M) {
+            const int rid = p.z_group ? z * p.M + m : m;
+            const int src = (p.a_rows ? p.a_rows[rid] : rid) / p.a_div;
+            arow[m] = A + (long long)src * p.lda;
+        }
+    }
+    const bf16_t* w0 = B + (long long)n0 * p.ldb;
+    const bf16_t* w1 = B + (long long)min(n0 + 1, p.N - 1) * p.ldb;
+    float acc0[MR], acc1[MR];
+#pragma unroll
+    for (int m = 0; m < MR; ++m) acc0[m] = acc1[m] = 0.0f;
+    const int kq = (((p.K + 3) / 4) + 7) & ~7;  // a wave's quarter of K, a multiple of 8
+    const int k_lo = wave * kq, k_hi = min(p.K, k_lo + kq);
+    constexpr int U = 2;
+    for (int k = k_lo + lane * 8; k < k_hi; k += 512 * U) {
+        float wa[U][8], wb[U][8];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            load_w8(w0, k + 512 * u, k_hi, p.b_vec, wa[u]);
+            load_w8(w1, k + 512 * u, k_hi, p.b_vec, wb[u]);
+        }
+#pragma unroll
+        for (int m = 0; m < MR; ++m) {
+            float s0 = acc0[m], s1 = acc1[m];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int kk = k + 512 * u;
+                f32x4 a0 = load_a4(arow[m], kk, k_hi, p.a_vec), a1 = load_a4(arow[m], kk + 4, k_hi, p.a_vec);
+                if (p.a_glu > 0 && arow[m]) {  // rows [gate | up]: silu(gate) * up
+                    const f32x4 u0 = load_a4(arow[m] + p.a_glu, kk, k_hi, p.a_vec && p.a_glu % 4 == 0);
+                    const f32x4 u1 = load_a4(arow[m] + p.a_glu, kk + 4, k_hi, p.a_vec && p.a_glu % 4 == 0);
+                    a0.x = a0.x / (1.0f + expf(-a0.x)) * u0.x; a0.y = a0.y / (1.0f + expf(-a0.y)) * u0.y;
+                    a0.z = a0.z / (1.0f + expf(-a0.z)) * u0.z; a0.w = a0.w / (1.0f + expf(-a0.w)) * u0.w;
+                    a1.x = a1.x / (1.0f + expf(-a1.x)) * u1.x; a1.y = a1.y / (1.0f + expf(-a1.y)) * u1.y;
+                    a1.z = a1.z / (1.0f + expf(-a1.z)) * u1.z; a1.w = a1.w / (1.0f + expf(-a1.w)) * u1.w;
+                }
+                s0 = fmaf(a0.x, wa[u][0], s0); s1 = fmaf(a0.x, wb[u][0], s1);
+                s0 = fmaf(a0.y, wa[u][1], s0); s1 = fmaf(a0.y, wb[u][1], s1);
+                s0 = fmaf(a0.z, wa[u][2], s0); s1 = fmaf(a0.z, wb[u][2], s1);
+                s0 = fmaf(a0.w, wa[u][3], s0); s1 = fmaf(a0.w, wb[u][3], s1);
+                s0 = fmaf(a1.x, wa[u][4], s0); s1 = fmaf(a1.x, wb[u][4], s1);
+                s0 = fmaf(a1.y, wa[u][5], s0); s1 = fmaf(a1.y, wb[u][5], s1);
+                s0 = fmaf(a1.z, wa[u][6], s0); s1 = fmaf(a1.z, wb[u][6], s1);
+                s0 = fmaf(a1.w, wa[u][7], s0); s1 = fmaf(a1.w, wb[u][7], s1);
+            }
+            acc0[m] = s0;
+            acc1[m] = s1;
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < MR; ++m) {
+        const float t0 = wave_allsum(acc0[m]), t1 = wave_allsum(acc1[m]);
+        if (lane == 0) {
+            s_part[wave][m][0] = t0;
+            s_part[wave][m][1] = t1;
+        }
+    }
+    __syncthreads();
+    if (threadIdx.x < MR * 2) {
+        const int m = threadIdx.x >> 1, c = threadIdx.x & 1;
+        if (m < p.M && n0 + c < p.N)
+            C[(long long)m * p.ldc + n0 + c] = apply_act((s_part[0][m][c] + s_part[1][m][c]) + (s_part[2][m][c] + s_part[3][m][c]), p.act);
+    }
+}
+
 // ------------------------------------------------------------------------------------------------ matrix cores
 template <bool F32>
 struct Tile {
@@ -343,6 +424,14 @@ int launch_linear(const Linear& L, bool f32, hipStream_t s) {
     p.a_vec = ((reinterpret_cast<uintptr_t>(L.A) & 15) == 0 && L.lda % 4 == 0 && L.a_zoff % 4 == 0) ? 1 : 0;
     p.b_vec = ((reinterpret_cast<uintptr_t>(L.B) & 15) == 0 && L.ldb % 8 == 0 && L.b_zoff % 8 == 0) ? 1 : 0;
     if (!L.grp_off && L.M <= kGemvMaxRows) {
+        if (L.K >= 1024 && L.M <= 2) {  // long rows, one or two of them: K split over the waves, two weight rows per workgroup
+            const dim3 gks((L.N + 1) / 2, 1, L.nz);  // (from four rows on the activations are re-read by too many workgroups: measured slower)
+            if (L.M == 1) lm_gemv_ks_kernel<1><<<gks, 256, 0, s>>>(p);
+            else lm_gemv_ks_kernel<2><<<gks, 256, 0, s>>>(p);
+            note_kernel("lm_gemv_ks_kernel<%d>", L.M);
+            ZG_HIP(hipGetLastError());
+            return ZG_OK;
+        }
         const dim3 grid((L.N + 7) / 8, 1, L.nz);
         if (L.M == 1) lm_gemv_kernel<1><<<grid, 256, 0, s>>>(p);
         else if (L.M == 2) lm_gemv_kernel<2><<<grid, 256, 0, s>>>(p);
