@@ -351,7 +351,9 @@ def _checkpoint(tmp_path, cfg, w):
     d = tmp_path / "ckpt"
     d.mkdir()
     (d / "config.json").write_text(json.dumps(cfg))
-    weights_io.write_safetensors(str(d / "model.safetensors"), w)
+    extra = dict(w)
+    extra["positions.table"] = np.arange(6, dtype=np.int32)  # not a tensor of the configuration: every front end leaves it alone
+    weights_io.write_safetensors(str(d / "model.safetensors"), extra)
     return str(d)
 
 

@@ -256,7 +256,9 @@ inline void load_safetensors(zg_lm* g, const std::string& path) {
                 buf[i] = s ? -v : v;
             }
         }
-        if (zg_lm_load_tensor(g, kv.first.c_str(), buf.data(), count) != ZG_OK) throw std::runtime_error(std::string("load: ") + zg_last_error());
+        const int st = zg_lm_load_tensor(g, kv.first.c_str(), buf.data(), count);
+        if (st == ZG_ERR_ARG && strstr(zg_last_error(), "has no tensor")) continue;  // not a tensor of this configuration: left alone
+        if (st != ZG_OK) throw std::runtime_error(std::string("load: ") + zg_last_error());
     }
     size_t missing = 0;
     char names[512];

@@ -177,7 +177,12 @@ class LayeredLM:
         from . import weights_io
 
         m = cls(LMConfig.from_dir(path), dtype=dtype, **kw)
-        m.load_weights(weights_io.load_safetensors_f32(os.path.join(path, "model.safetensors")))
+        # tensors the configuration does not name are left alone (a checkpoint may carry tables of other tools); every tensor it
+        # does name must be there
+        m.load_weights(weights_io.load_safetensors_f32(os.path.join(path, "model.safetensors")), strict=False)
+        missing = m.missing_tensors()
+        if missing:
+            raise KeyError(f"{path}: {len(missing)} tensors missing from the checkpoint: {' '.join(missing[:8])}")
         return m
 
     def close(self):
