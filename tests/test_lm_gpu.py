@@ -290,6 +290,19 @@ def test_long_rows_in_decode_steps():
         m.close()
 
 
+def test_rows_wider_than_the_register_kernels():
+    """A width beyond what the one-round-trip norm kernels hold in registers: the general norm kernels and the unfused pass tail."""
+    cfg = tl.config([tl.hgrn2_layer(heads=1, dim=8, vdim=8, mlp=tl.moe_mlp(ff=8, experts=3, top=2)),
+                     tl.latent_layer(heads=1, dim=8, vdim=8, rot_dim=4, kv_rank=16, q_rank=8, mlp=tl.dense_mlp(ff=16))], vocab=61, width=4100)
+    w = tl.weights(cfg, seed=20)
+    toks = tl.tokens(64, 12, cfg["vocab"])
+    ref = lm_oracle.Model(cfg, w).forward(toks)[0]
+    m = make(cfg, w, "float32", max_tokens=64, max_seqs=2)
+    tl.assert_close(run_whole(m, toks), ref, "float32")
+    tl.assert_close(run_cut(m, toks, [2, 3, 4, 5, 6, 7, 8, 9]), ref, "float32")
+    m.close()
+
+
 def test_greedy_and_sampled_generation():
     cfg = full_cfg(loop={"start": 1, "stop": 3, "times": 2})
     w = tl.weights(cfg, seed=14, head_std=1.0)
