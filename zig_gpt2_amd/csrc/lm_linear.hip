@@ -443,11 +443,11 @@ int launch_linear(const Linear& L, bool f32, hipStream_t s) {
     }
     ZG_REQUIRE(L.a_glu == 0, ZG_ERR_ARG, "linear: the gated activation on load is for steps of few rows");
     ZG_REQUIRE(!(L.z_group && L.grp_off), ZG_ERR_ARG, "linear: a matrix per batch and row groups exclude each other");
-    auto tiles = [&](int b) { return (long long)((L.M + b - 1) / b + (L.grp_off ? L.n_groups : 0)) * ((L.N + b - 1) / b) * L.nz; };
-    // 128 x 128 tiles once they fill the chip twice over; ZGPT2_LM_GEMM_TILE=64|128 pins the choice (tests run small shapes
-    // through the large tiles with it)
-    bool big = tiles(128) >= 512;
-    if (const char* e = getenv("ZGPT2_LM_GEMM_TILE")) big = atoi(e) == 128 ? true : atoi(e) == 64 ? false : big;
+    // 64 x 64 tiles.  The 128 x 128 form of the same kernel measured slower at every size tried (a prompt pass of 8 x 1023
+    // tokens at width 1600: 143 against 127 ms; width 768: 14.6 against 12.9 ms) and is kept behind ZGPT2_LM_GEMM_TILE=128 only
+    // (tests run ragged shapes through it).
+    bool big = false;
+    if (const char* e = getenv("ZGPT2_LM_GEMM_TILE")) big = atoi(e) == 128;
     const int b = big ? 128 : 64;
     const dim3 grid((L.N + b - 1) / b, (L.M + b - 1) / b + (L.grp_off ? L.n_groups : 0), L.nz);
     ZG_REQUIRE(grid.y <= 65535 && grid.z <= 65535, ZG_ERR_UNSUPPORTED, "linear: %d rows in %d batches exceed the grid", L.M, L.nz);
