@@ -270,9 +270,9 @@ def test_large_tiles_on_small_shapes(monkeypatch):
 
 
 def test_long_rows_in_decode_steps():
-    """Feed-forward widths beyond 1024: decode steps multiply their down-projections with K split over the waves of a workgroup
+    """Feed-forward widths beyond 1536: decode steps multiply their down-projections with K split over the waves of a workgroup
     (one width a multiple of the 16-byte pieces, one not) alone and as a batch of two; a batch of three takes the general kernel."""
-    cfg = tl.config([tl.hgrn2_layer(mlp=tl.dense_mlp(ff=1100)), tl.latent_layer(mlp=tl.dense_mlp(ff=1032))])
+    cfg = tl.config([tl.hgrn2_layer(mlp=tl.dense_mlp(ff=1620)), tl.latent_layer(mlp=tl.dense_mlp(ff=1544))])
     w = tl.weights(cfg, seed=19)
     oracle = lm_oracle.Model(cfg, w)
     toks = [tl.tokens(63 + i, 14, cfg["vocab"]) for i in range(3)]

@@ -148,7 +148,7 @@ __global__ __launch_bounds__(256) void lm_gemv_kernel(const LinArgs p) {
     }
 }
 
-// The same for long rows (K >= 1024): a workgroup owns two weight rows and its four waves split K into quarters, so a matrix of
+// The same for long rows (K >= 1536; at 1024 columns half the lanes of a quarter idle and it measured 6 % slower): a workgroup owns two weight rows and its four waves split K into quarters, so a matrix of
 // a few MB is requested whole in one go by thousands of waves instead of trip by trip by a few hundred (a 1600 x 1600 matrix:
 // 800 workgroups, every 16-byte piece in flight at once); the quarter sums meet in the LDS.  The summation order of an output
 // depends on K alone.
@@ -424,7 +424,7 @@ int launch_linear(const Linear& L, bool f32, hipStream_t s) {
     p.a_vec = ((reinterpret_cast<uintptr_t>(L.A) & 15) == 0 && L.lda % 4 == 0 && L.a_zoff % 4 == 0) ? 1 : 0;
     p.b_vec = ((reinterpret_cast<uintptr_t>(L.B) & 15) == 0 && L.ldb % 8 == 0 && L.b_zoff % 8 == 0) ? 1 : 0;
     if (!L.grp_off && L.M <= kGemvMaxRows) {
-        if (L.K >= 1024 && L.M <= 2) {  // long rows, one or two of them: K split over the waves, two weight rows per workgroup
+        if (L.K >= 1536 && L.M <= 2 && L.nz <= 4) {  // long rows, one or two of them, few batches: K split over the waves, two weight rows per workgroup
             const dim3 gks((L.N + 1) / 2, 1, L.nz);  // (from four rows on the activations are re-read by too many workgroups: measured slower)
             if (L.M == 1) lm_gemv_ks_kernel<1><<<gks, 256, 0, s>>>(p);
             else lm_gemv_ks_kernel<2><<<gks, 256, 0, s>>>(p);
