@@ -346,15 +346,36 @@ int zg_gpt_generate_fetch_many(zg_gpt* const* handles, size_t n_handles, size_t 
  * architecture maps to which layer list is the host program's business (zig_gpt2_amd/models.py, zig_gpt2_amd/lm.py).
  *
  * A layer computes   x += norm1b(mixer(shift(norm1(x))));   x += norm2b(ff(norm2(x)))
- * with RMS norms whose stored weight is an offset from one, and shift(h)_t = h_t + (h_(t-1) - h_t) * mu.
+ * with RMS norms whose stored weight is an offset from one, and shift(h)_t = h_t + (h_(t-1) - h_t) * mu — or, with
+ * canon_taps >= 1,   x += norm1b(mixer(c1(norm1(x))));   x += norm2b(ff(c2(norm2(x))))   with c(h) = h + conv(h).
  * Norms, softmax, router, gates, recurrent state, positions and the residual are fp32; matrix products take bf16 operands with
  * fp32 accumulation, or true fp32 products under ZG_LM_F32.  Weights are stored bf16. */
 enum {
     ZG_LM_MIX_HGRN2 = 1,            /* gated linear recurrence: S = diag(f) S + (1 - f) v^T, o = S^T q, f bounded from below */
-    ZG_LM_MIX_LATENT_ATTENTION = 2  /* causal softmax attention whose keys and values are up-projections of a cached latent, plus
+    ZG_LM_MIX_LATENT_ATTENTION = 2, /* causal softmax attention whose keys and values are up-projections of a cached latent, plus
                                        one rotary key part shared by the heads; queries through a latent of their own */
+    ZG_LM_MIX_PARALLEL = 3,         /* two branches on the same input, each RMS-normed over the width, half their sum:
+                                       left   grouped-query softmax attention inside a sliding window, with a learned sink in the
+                                              denominator, the heads' weights mixed by a [heads, heads] matrix, rotary on q / k (first
+                                              rot_dims channels, interleaved pairs) and VALUES rotated by their position over all vdim
+                                              channels, the head's output turned back by the query's position;
+                                       right  a real-gated linear recurrent unit behind a short causal convolution:
+                                              a = exp(-8 r softplus(lam)), S = a S + sqrt(1 - a^2) i u, out = S * gelu_tanh(y) */
+    ZG_LM_MIX_CHANNEL_DELTA = 4     /* gated delta rule with a decay per key channel: S = diag(g) S; u = beta (v - S^T k);
+                                       S += k u^T; o = S^T q;  q, k, v behind short causal convolutions + silu, q and k of unit
+                                       length, the decay and the output gate through two-step (low-rank) projections */
 };
-enum { ZG_LM_FF_NONE = 0, ZG_LM_FF_DENSE = 1 /* down(relu(up h)^2) */, ZG_LM_FF_MOE = 2 /* top-k of `experts` gated units */ };
+enum { ZG_LM_FF_NONE = 0, ZG_LM_FF_DENSE = 1 /* down(relu(up h)^2) */, ZG_LM_FF_MOE = 2 /* top-k of `experts` units */ };
+/* Activation of an expert (ff_act) and the rule of the router (router) of ZG_LM_FF_MOE. */
+enum {
+    ZG_LM_ACT_GLU_SILU = 0, /* down(silu(gate h) * up h): tensors e<j>.gate / up / down */
+    ZG_LM_ACT_GELU = 1      /* down(gelu(up h)), the exact (erf) form: tensors e<j>.up / down */
+};
+enum {
+    ZG_LM_ROUTE_SOFTMAX_ALL = 0, /* s = softmax over all experts; the `top` largest s + correction; weights s */
+    ZG_LM_ROUTE_TOP_LOGITS = 1   /* z = router h + bias (`router.b`); the `top` largest z; weights softmax over the chosen z */
+};
+enum { ZG_LM_ROT_PLAIN = 0, ZG_LM_ROT_YARN = 1 /* blend by pair index, amplitude factor */, ZG_LM_ROT_BANDS = 2 /* by wavelength: see rot_* */ };
 typedef struct {
     int mixer;                    /* ZG_LM_MIX_* */
     int heads, dim, vdim;         /* both mixers: heads, key (unrotated) channels and value channels per head */
@@ -362,15 +383,25 @@ typedef struct {
     float scale;                  /* latent attention: factor of the scores */
     int rot_dims;                 /* rotary: how many of the rot_dim channels are rotated (interleaved pairs) */
     float rot_base;
-    int rot_scaled;               /* != 0: YaRN blend of the frequencies with the four constants below */
+    int rot_scaled;               /* ZG_LM_ROT_*: YARN blends the frequencies with the four constants below; BANDS keeps a frequency whose
+                                     wavelength is below original / rot_fast, divides it by factor above original / rot_slow, and
+                                     blends linearly in (original / wavelength) between */
     float rot_factor, rot_original, rot_fast, rot_slow;
     int ff;                       /* ZG_LM_FF_* */
     int ff_width;                 /* hidden width of the dense feed-forward, or of ONE expert */
     int experts, top;
+    int kv_heads;                 /* parallel / delta rule: key heads, each shared by heads / kv_heads heads (0: = heads) */
+    int window;                   /* parallel: a position sees itself and the window - 1 positions before it (0: all before it) */
+    int lru_width, lru_blocks, lru_conv; /* parallel: channels of the recurrent unit, blocks of its gate matrices, taps of its convolution */
+    int conv;                     /* delta rule: taps of the convolutions on q, k, v */
+    int decay_rank, gate_rank;    /* delta rule: inner sizes of the two-step projections of the decay and of the output gate */
+    int ff_act, router;           /* ZG_LM_ACT_*, ZG_LM_ROUTE_* */
 } zg_lm_layer;
 enum {
     ZG_LM_F32 = 1 << 0,     /* true 32-bit products everywhere */
-    ZG_LM_NO_GRAPH = 1 << 1 /* launch the kernels of a decode step one by one instead of replaying the hipGraph captured for its batch size */
+    ZG_LM_NO_GRAPH = 1 << 1, /* launch the kernels of a decode step one by one instead of replaying the hipGraph captured for its batch size */
+    ZG_LM_TIED_HEAD = 1 << 2, /* logits = embed . norm(x): there is no `head` tensor */
+    ZG_LM_LOOP_READD = 1 << 3 /* every repetition of the looped span but the first starts by adding the embedding output to x */
 };
 typedef struct {
     size_t vocab, width, n_layers;
@@ -382,14 +413,20 @@ typedef struct {
     size_t max_step_tokens; /* rows of one pass; a longer step is cut into portions (0: 2048) */
     size_t page_tokens;     /* tokens per cache page (0: 64) */
     unsigned flags;         /* ZG_LM_* */
+    float embed_scale;      /* x = embed[token] * embed_scale (0: 1) */
+    int canon_taps;         /* 0: the sublayer input of the mixer is the token shift (tensor `shift`).  >= 1: BOTH sublayers read
+                               h + conv(h), a causal convolution per channel over the last canon_taps tokens (tensors `canon1`,
+                               `canon2` [width][taps], last column = the current token); a slot keeps the taps - 1 last inputs */
 } zg_lm_config;
 typedef struct zg_lm zg_lm;
 /* One arena for weights, state and scratch; the handle owns a stream on `device`.  Needs no zg_init. */
 int zg_lm_create(zg_lm** out, const zg_lm_config* config, int device);
 int zg_lm_destroy(zg_lm* g);
-/* Weights by checkpoint name: `embed`, `head`, `final.norm`, and per layer i `l<i>.norm1|norm1b|norm2|norm2b|shift`,
- * `l<i>.mix.*` (hgrn2: q f f.b lower v norm o; latent attention: dq dq.norm uq dkv dkv.norm uk uv o) and `l<i>.mlp.*`
- * (dense: up down; experts: e<j>.gate e<j>.up e<j>.down router correction).  data: fp32 on the host, `len` elements, matrices
+/* Weights by checkpoint name: `embed`, `head`, `final.norm`, and per layer i `l<i>.norm1|norm1b|norm2|norm2b|shift|canon1|canon2`,
+ * `l<i>.mix.*` (hgrn2: q f f.b lower v norm o; latent attention: dq dq.norm uq dkv dkv.norm uk uv o; parallel: left.q left.k
+ * left.v left.sink left.talk left.o left.out right.y right.y.b right.x right.x.b right.conv right.conv.b right.ra right.ra.b
+ * right.ri right.ri.b right.lam right.o right.out; delta rule: q q.conv k k.conv v v.conv b A_log dt_bias a1 a2 g1 g2 norm o)
+ * and `l<i>.mlp.*` (dense: up down; experts: e<j>.gate e<j>.up e<j>.down router, and correction or router.b).  data: fp32 on the host, `len` elements, matrices
  * [out][in] row-major; matrices are stored bf16 (round to nearest even).  ZG_ERR_ARG for a name the configuration does not have. */
 int zg_lm_load_tensor(zg_lm* g, const char* name, const float* data, size_t len);
 /* How many tensors of the configuration have not been loaded; names_out (may be NULL) receives them, space separated. */

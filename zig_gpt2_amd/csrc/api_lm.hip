@@ -11,6 +11,12 @@
 //       latent cache per attention pass [page][token][kv_rank + rot_dim] ]          all fp32
 //   [ scratch of one portion (max_step_tokens rows) | step metadata | logits ]
 //
+// Designs whose sublayers read h + conv(h) (canon_taps >= 1) and the mixers with convolutions or recurrences of their own keep, per
+// slot and layer pass, one block of fp32 state: the tails of the input convolutions (the taps - 1 last inputs of both sublayers),
+// the tail of the mixer's short convolutions, and its recurrent state (a vector per channel, or a matrix per head).  Windowed
+// attention caches rotated keys and rotated values per token in the paged cache, through the same page table as the latents;
+// pages that every attention pass's window has left behind return to the pool while the sequence is still open.
+//
 // Latent attention runs in its absorbed form in prompts and in decoding alike: score_j = (W_uk^T q_nope) . c_j + q_rot . k_rot_j,
 // out = W_uv (sum_j p_j c_j) — only the latent c_j and the rotated key part are cached, and a portion of a prompt needs nothing
 // of the tokens before it but their cache rows.
@@ -52,19 +58,35 @@ struct LayerW {
     float *dq_norm = nullptr, *dkv_norm = nullptr, *rot_freq = nullptr;
     float rot_amp = 1.0f;
     bf16_t *up = nullptr, *down = nullptr, *gu = nullptr, *edown = nullptr, *router = nullptr;
-    float* correction = nullptr;
+    float* correction = nullptr;  // the router's correction of the choice, or its bias (ZG_LM_ROUTE_TOP_LOGITS)
+    // input convolutions of the two sublayers ([W][taps] fp32)
+    float *canon1 = nullptr, *canon2 = nullptr;
+    // parallel / delta rule: one fused projection (parallel: q | k | v | y | x;  delta rule: q | k | v | b | a1 | g1)
+    bf16_t* wcat = nullptr;
+    int n_cat = 0;
+    // parallel
+    bf16_t *ro = nullptr, *ra = nullptr, *ri = nullptr;
+    float *sink = nullptr, *talk = nullptr, *left_out = nullptr, *right_out = nullptr, *yb = nullptr, *xb = nullptr, *convw = nullptr, *convb = nullptr;
+    float *rab = nullptr, *rib = nullptr, *lam = nullptr, *vfreq = nullptr;
+    // delta rule
+    bf16_t *a2 = nullptr, *g2 = nullptr;
+    float *a_log = nullptr, *dt_bias = nullptr;
 };
 
 struct Pass {
     int layer = 0;
     size_t hgrn_off = 0;     // floats into a slot's recurrent-state block
-    float* cache = nullptr;  // latent cache of this pass
+    float* cache = nullptr;  // latent cache (or key / value cache) of this pass
+    bool readd = false;      // the embedding output is added to x in front of this pass
+    // floats into a slot's block of sequence state: tails of the two input convolutions, tail of the mixer's own convolution,
+    // the mixer's recurrent state
+    size_t canon1_off = 0, canon2_off = 0, conv_off = 0, rec_off = 0;
 };
 
 struct Slot {
     bool open = false;
     size_t len = 0;
-    std::vector<int> pages;
+    std::vector<int> pages;  // by position / page_tokens; -1: returned to the pool (behind every window)
 };
 
 struct Bump {
@@ -139,6 +161,11 @@ struct zg_lm {
     float* shift_state = nullptr;  // [NS][passes][W]
     float* hgrn_state = nullptr;   // [NS][hgrn_floats]
     size_t hgrn_floats = 0;
+    float* seq_state = nullptr;  // [NS][seq_floats]: convolution tails and recurrent states of the passes that have them
+    size_t seq_floats = 0;
+    int canon = 0;        // taps of the sublayers' input convolution (0: token shift)
+    int keep_tokens = 0;  // > 0: no attention pass looks further back than this many tokens
+    float embed_scale = 1.0f;
     int* page_table = nullptr;  // [NS][max_pages]
     std::vector<Slot> slots;
     std::vector<int> free_pages;
@@ -148,6 +175,7 @@ struct zg_lm {
     float *row_max = nullptr, *samp_ws = nullptr, *samp_u = nullptr, *amax_val = nullptr;
     int* amax_idx = nullptr;
     float *attn_ws = nullptr, *scan_ws = nullptr;
+    float *x0 = nullptr, *hc = nullptr, *y2 = nullptr, *ta = nullptr, *tb = nullptr, *tc = nullptr, *td = nullptr;
     size_t scan_ws_floats = 0;
     size_t attn_ws_floats = 0;
     int *pick = nullptr, *grp_off = nullptr, *sorted = nullptr, *inv = nullptr, *tok_out = nullptr, *flag = nullptr;
@@ -165,7 +193,9 @@ struct zg_lm {
 
 namespace {
 
-size_t meta_ints(const zg_lm* g) { return (size_t)6 * g->MS + (size_t)3 * g->NS; }
+// ids | pos | slot | prev | last-entry | want rows | entry start | entry len | entry slot | place of the row inside its entry
+size_t meta_ints(const zg_lm* g) { return (size_t)7 * g->MS + (size_t)3 * g->NS; }
+size_t meta_row_off(const zg_lm* g) { return (size_t)6 * g->MS + (size_t)3 * g->NS; }
 
 // Everything that lives in the arena, in one place: called once with a null base to measure and once to place.
 void layout(zg_lm* g, Bump& b) {
@@ -191,11 +221,25 @@ void layout(zg_lm* g, Bump& b) {
         t.init = init;
         T[name] = t;
     };
+    auto vec_at = [&](const std::string& name, float* base, size_t off, size_t n, int init) {
+        Tensor t;
+        t.dev = base ? base + off : nullptr;
+        t.rows = 1;
+        t.cols = n;
+        t.init = init;
+        T[name] = t;
+    };
+    const size_t taps = g->canon;
     g->embed = b.take<bf16_t>(V * W);
     mat("embed", g->embed, 0, V, W);
-    g->head = b.take<bf16_t>(V * W);
-    mat("head", g->head, 0, V, W);
+    if (g->cfg.flags & ZG_LM_TIED_HEAD) {
+        g->head = g->embed;
+    } else {
+        g->head = b.take<bf16_t>(V * W);
+        mat("head", g->head, 0, V, W);
+    }
     vec("final.norm", g->final_norm, W, INIT_OFFSET);
+    size_t max_t = 1;
     size_t max_proj = 1, max_qr = 1, max_q = 1, max_qa = 1, max_ctx = 1, max_o = 1, max_ff = 1, max_assign = 1, max_gu = 1, max_hb = 1, max_e = 1, max_att_part = 0, max_scan = 0;
     for (size_t i = 0; i < g->layers.size(); ++i) {
         LayerW& L = g->layers[i];
@@ -203,9 +247,70 @@ void layout(zg_lm* g, Bump& b) {
         const std::string p = "l" + std::to_string(i) + ".";
         vec(p + "norm1", L.norm1, W, INIT_OFFSET);
         vec(p + "norm1b", L.norm1b, W, INIT_OFFSET);
-        vec(p + "shift", L.shift, W, INIT_UNIT);
+        if (taps == 0) vec(p + "shift", L.shift, W, INIT_UNIT);
+        else vec(p + "canon1", L.canon1, W * taps, INIT_OFFSET);
         const size_t H = d.heads, D = d.dim, Vd = d.vdim;
-        if (d.mixer == ZG_LM_MIX_HGRN2) {
+        if (d.mixer == ZG_LM_MIX_PARALLEL) {
+            const size_t G = d.kv_heads, C = d.lru_width, NB = d.lru_blocks, BS = C / NB, HV = H * Vd;
+            const size_t NP = H * D + G * D + G * Vd + 2 * C;
+            L.n_cat = (int)NP;
+            L.wcat = b.take<bf16_t>(NP * W);
+            mat(p + "mix.left.q", L.wcat, 0, H * D, W);
+            mat(p + "mix.left.k", L.wcat, H * D, G * D, W);
+            mat(p + "mix.left.v", L.wcat, H * D + G * D, G * Vd, W);
+            mat(p + "mix.right.y", L.wcat, H * D + G * D + G * Vd, C, W);
+            mat(p + "mix.right.x", L.wcat, H * D + G * D + G * Vd + C, C, W);
+            vec(p + "mix.left.sink", L.sink, H, INIT_OFFSET);
+            vec(p + "mix.left.talk", L.talk, H * H, INIT_UNIT);
+            L.o = b.take<bf16_t>(W * HV);
+            mat(p + "mix.left.o", L.o, 0, W, HV);
+            vec(p + "mix.left.out", L.left_out, W, INIT_PLAIN);
+            vec(p + "mix.right.out", L.right_out, W, INIT_PLAIN);
+            vec(p + "mix.right.y.b", L.yb, C, INIT_OFFSET);
+            vec(p + "mix.right.x.b", L.xb, C, INIT_OFFSET);
+            vec(p + "mix.right.conv", L.convw, C * d.lru_conv, INIT_OFFSET);
+            vec(p + "mix.right.conv.b", L.convb, C, INIT_OFFSET);
+            L.ra = b.take<bf16_t>(NB * BS * BS);
+            mat(p + "mix.right.ra", L.ra, 0, NB * BS, BS);
+            L.ri = b.take<bf16_t>(NB * BS * BS);
+            mat(p + "mix.right.ri", L.ri, 0, NB * BS, BS);
+            vec(p + "mix.right.ra.b", L.rab, C, INIT_OFFSET);
+            vec(p + "mix.right.ri.b", L.rib, C, INIT_OFFSET);
+            vec(p + "mix.right.lam", L.lam, C, INIT_OFFSET);
+            L.ro = b.take<bf16_t>(W * C);
+            mat(p + "mix.right.o", L.ro, 0, W, C);
+            L.rot_freq = b.take<float>(std::max<size_t>(1, d.rot_dims / 2));
+            L.vfreq = b.take<float>(std::max<size_t>(1, Vd / 2));
+            max_proj = std::max(max_proj, NP);
+            max_o = std::max(max_o, HV);
+            max_t = std::max(max_t, C);
+        } else if (d.mixer == ZG_LM_MIX_CHANNEL_DELTA) {
+            const size_t G = d.kv_heads, HV = H * Vd, CC = 2 * G * D + HV, RA = d.decay_rank, RG = d.gate_rank;
+            const size_t NP = CC + H + RA + RG;
+            L.n_cat = (int)NP;
+            L.wcat = b.take<bf16_t>(NP * W);
+            mat(p + "mix.q", L.wcat, 0, G * D, W);
+            mat(p + "mix.k", L.wcat, G * D, G * D, W);
+            mat(p + "mix.v", L.wcat, 2 * G * D, HV, W);
+            mat(p + "mix.b", L.wcat, CC, H, W);
+            mat(p + "mix.a1", L.wcat, CC + H, RA, W);
+            mat(p + "mix.g1", L.wcat, CC + H + RA, RG, W);
+            L.convw = b.take<float>(CC * d.conv);
+            vec_at(p + "mix.q.conv", L.convw, 0, G * D * d.conv, INIT_OFFSET);
+            vec_at(p + "mix.k.conv", L.convw, G * D * d.conv, G * D * d.conv, INIT_OFFSET);
+            vec_at(p + "mix.v.conv", L.convw, 2 * G * D * d.conv, HV * d.conv, INIT_OFFSET);
+            L.a2 = b.take<bf16_t>(H * D * RA);
+            mat(p + "mix.a2", L.a2, 0, H * D, RA);
+            L.g2 = b.take<bf16_t>(HV * RG);
+            mat(p + "mix.g2", L.g2, 0, HV, RG);
+            vec(p + "mix.A_log", L.a_log, H, INIT_OFFSET);
+            vec(p + "mix.dt_bias", L.dt_bias, H * D, INIT_OFFSET);
+            vec(p + "mix.norm", L.hnorm, Vd, INIT_PLAIN);
+            L.o = b.take<bf16_t>(W * HV);
+            mat(p + "mix.o", L.o, 0, W, HV);
+            max_proj = std::max(max_proj, NP);
+            max_t = std::max(max_t, std::max(CC, std::max(H * D, HV)));
+        } else if (d.mixer == ZG_LM_MIX_HGRN2) {
             const size_t HD = H * D, HV = H * Vd;
             L.qfv = b.take<bf16_t>((2 * HD + HV) * W);
             mat(p + "mix.q", L.qfv, 0, HD, W);
@@ -246,6 +351,7 @@ void layout(zg_lm* g, Bump& b) {
         if (d.ff != ZG_LM_FF_NONE) {
             vec(p + "norm2", L.norm2, W, INIT_OFFSET);
             vec(p + "norm2b", L.norm2b, W, INIT_OFFSET);
+            if (taps) vec(p + "canon2", L.canon2, W * taps, INIT_OFFSET);
         }
         const size_t F = d.ff_width;
         if (d.ff == ZG_LM_FF_DENSE) {
@@ -255,20 +361,20 @@ void layout(zg_lm* g, Bump& b) {
             mat(p + "mlp.down", L.down, 0, W, F);
             max_ff = std::max(max_ff, F);
         } else if (d.ff == ZG_LM_FF_MOE) {
-            const size_t E = d.experts;
-            L.gu = b.take<bf16_t>(E * 2 * F * W);
+            const size_t E = d.experts, UF = d.ff_act == ZG_LM_ACT_GLU_SILU ? 2 * F : F;  // rows of an expert's first matrix
+            L.gu = b.take<bf16_t>(E * UF * W);
             L.edown = b.take<bf16_t>(E * W * F);
             for (size_t e = 0; e < E; ++e) {
                 const std::string q = p + "mlp.e" + std::to_string(e) + ".";
-                mat(q + "gate", L.gu, e * 2 * F, F, W);
-                mat(q + "up", L.gu, e * 2 * F + F, F, W);
+                if (UF == 2 * F) mat(q + "gate", L.gu, e * 2 * F, F, W);
+                mat(q + "up", L.gu, e * UF + (UF - F), F, W);
                 mat(q + "down", L.edown, e * W, W, F);
             }
             L.router = b.take<bf16_t>(E * W);
             mat(p + "mlp.router", L.router, 0, E, W);
-            vec(p + "mlp.correction", L.correction, E, INIT_OFFSET);
+            vec(p + (d.router == ZG_LM_ROUTE_TOP_LOGITS ? "mlp.router.b" : "mlp.correction"), L.correction, E, INIT_OFFSET);
             max_assign = std::max(max_assign, (size_t)d.top);
-            max_gu = std::max(max_gu, (size_t)d.top * 2 * F);
+            max_gu = std::max(max_gu, (size_t)d.top * UF);
             max_hb = std::max(max_hb, (size_t)d.top * F);
             max_e = std::max(max_e, E);
         }
@@ -285,15 +391,48 @@ void layout(zg_lm* g, Bump& b) {
     }
     g->hgrn_floats = hg;
     g->hgrn_state = b.take<float>(std::max<size_t>(1, NS * hg));
+    size_t sq = 0;
+    for (Pass& ps : g->passes) {
+        const zg_lm_layer& d = g->layers[ps.layer].d;
+        if (taps > 1) {
+            ps.canon1_off = sq;
+            sq += (taps - 1) * W;
+            if (d.ff != ZG_LM_FF_NONE) {
+                ps.canon2_off = sq;
+                sq += (taps - 1) * W;
+            }
+        }
+        if (d.mixer == ZG_LM_MIX_PARALLEL) {
+            ps.conv_off = sq;
+            sq += (size_t)(d.lru_conv - 1) * d.lru_width;
+            ps.rec_off = sq;
+            sq += d.lru_width;
+        } else if (d.mixer == ZG_LM_MIX_CHANNEL_DELTA) {
+            ps.conv_off = sq;
+            sq += (size_t)(d.conv - 1) * (2 * d.kv_heads * d.dim + d.heads * d.vdim);
+            ps.rec_off = sq;
+            sq += (size_t)d.heads * d.dim * d.vdim;
+        }
+    }
+    g->seq_floats = sq;
+    g->seq_state = b.take<float>(std::max<size_t>(1, NS * sq));
     g->page_table = b.take<int>(NS * g->max_pages);
     for (Pass& ps : g->passes) {
         const zg_lm_layer& d = g->layers[ps.layer].d;
         if (d.mixer == ZG_LM_MIX_LATENT_ATTENTION) ps.cache = b.take<float>((size_t)g->n_pages * g->P * (d.kv_rank + d.rot_dim));
+        if (d.mixer == ZG_LM_MIX_PARALLEL) ps.cache = b.take<float>((size_t)g->n_pages * g->P * d.kv_heads * (d.dim + d.vdim));
     }
     // scratch
     g->x = b.take<float>(MS * W);
     g->h = b.take<float>(MS * W);
     g->y = b.take<float>(MS * W);
+    g->x0 = b.take<float>(MS * W);
+    g->hc = b.take<float>(MS * W);
+    g->y2 = b.take<float>(MS * W);
+    g->ta = b.take<float>(MS * max_t);
+    g->tb = b.take<float>(MS * max_t);
+    g->tc = b.take<float>(MS * max_t);
+    g->td = b.take<float>(MS * max_t);
     g->proj = b.take<float>(MS * max_proj);
     g->cq = b.take<float>(MS * max_qr);
     g->q = b.take<float>(MS * max_q);
@@ -332,6 +471,21 @@ void rotary_table(const zg_lm_layer& d, std::vector<float>& freq, float& amp) {
     const int dims = d.rot_dims, half = dims / 2;
     freq.resize(std::max(1, half));
     amp = 1.0f;
+    if (d.rot_scaled == ZG_LM_ROT_BANDS) {  // by wavelength: short waves stay, long waves are slowed, a linear blend between
+        for (int i = 0; i < half; ++i) {
+            const double f = pow((double)d.rot_base, -2.0 * i / dims), wave = 2.0 * M_PI / f;
+            const double orig = d.rot_original, high = d.rot_fast, low = d.rot_slow;
+            double out = f;
+            if (wave < orig / high) out = f;
+            else if (wave > orig / low) out = f / d.rot_factor;
+            else {
+                const double t = (orig / wave - low) / (high - low);
+                out = (1.0 - t) * f / d.rot_factor + t * f;
+            }
+            freq[i] = (float)out;
+        }
+        return;
+    }
     double lo = 0, hi = 0;
     if (d.rot_scaled) {
         auto corr = [&](double t) { return dims * log((double)d.rot_original / (2.0 * M_PI * t)) / (2.0 * log((double)d.rot_base)); };
@@ -350,9 +504,26 @@ void rotary_table(const zg_lm_layer& d, std::vector<float>& freq, float& amp) {
 }
 
 int check_layer(const zg_lm_layer& d, size_t i) {
-    ZG_REQUIRE(d.mixer == ZG_LM_MIX_HGRN2 || d.mixer == ZG_LM_MIX_LATENT_ATTENTION, ZG_ERR_ARG, "layer %zu: unknown mixer %d", i, d.mixer);
+    ZG_REQUIRE(d.mixer >= ZG_LM_MIX_HGRN2 && d.mixer <= ZG_LM_MIX_CHANNEL_DELTA, ZG_ERR_ARG, "layer %zu: unknown mixer %d", i, d.mixer);
     ZG_REQUIRE(d.heads >= 1 && d.dim >= 1 && d.vdim >= 1, ZG_ERR_ARG, "layer %zu: heads %d dim %d vdim %d", i, d.heads, d.dim, d.vdim);
-    if (d.mixer == ZG_LM_MIX_HGRN2) {
+    if (d.mixer == ZG_LM_MIX_PARALLEL || d.mixer == ZG_LM_MIX_CHANNEL_DELTA)
+        ZG_REQUIRE(d.kv_heads >= 1 && d.heads % d.kv_heads == 0, ZG_ERR_ARG, "layer %zu: %d heads on %d key heads", i, d.heads, d.kv_heads);
+    if (d.mixer == ZG_LM_MIX_PARALLEL) {
+        ZG_REQUIRE(d.vdim % 2 == 0, ZG_ERR_ARG, "layer %zu: %d value channels per head cannot be rotated in pairs", i, d.vdim);
+        ZG_REQUIRE(d.rot_dims >= 0 && d.rot_dims % 2 == 0 && d.rot_dims <= d.dim, ZG_ERR_ARG, "layer %zu: %d rotated dimensions of %d", i, d.rot_dims,
+                   d.dim);
+        ZG_REQUIRE(d.rot_base > 0.0f && d.window >= 0, ZG_ERR_ARG, "layer %zu: rotary base %f, window %d", i, d.rot_base, d.window);
+        ZG_REQUIRE(!d.rot_scaled || (d.rot_factor > 0.0f && d.rot_original > 0.0f && d.rot_fast > 0.0f && d.rot_slow > 0.0f &&
+                                     (d.rot_scaled != ZG_LM_ROT_BANDS || d.rot_fast != d.rot_slow)),
+                   ZG_ERR_ARG, "layer %zu: rotary scaling constants", i);
+        ZG_REQUIRE(d.lru_width >= 1 && d.lru_blocks >= 1 && d.lru_width % d.lru_blocks == 0 && d.lru_conv >= 1 && d.lru_conv <= 16, ZG_ERR_ARG,
+                   "layer %zu: recurrent unit of %d channels in %d blocks, %d taps", i, d.lru_width, d.lru_blocks, d.lru_conv);
+    } else if (d.mixer == ZG_LM_MIX_CHANNEL_DELTA) {
+        ZG_REQUIRE(d.conv >= 1 && d.conv <= 16 && d.decay_rank >= 1 && d.gate_rank >= 1, ZG_ERR_ARG, "layer %zu: %d taps, inner sizes %d and %d", i,
+                   d.conv, d.decay_rank, d.gate_rank);
+        ZG_REQUIRE(d.dim <= 256 && d.vdim <= 256, ZG_ERR_UNSUPPORTED, "layer %zu: a delta-rule state of %d x %d per head (at most 256 each)", i, d.dim,
+                   d.vdim);
+    } else if (d.mixer == ZG_LM_MIX_HGRN2) {
         ZG_REQUIRE(d.dim <= 256, ZG_ERR_UNSUPPORTED, "layer %zu: %d key channels per head of the recurrence (at most 256)", i, d.dim);
     } else {
         ZG_REQUIRE(d.rot_dim >= 0 && d.kv_rank >= 1 && d.q_rank >= 1, ZG_ERR_ARG, "layer %zu: rot_dim %d kv_rank %d q_rank %d", i, d.rot_dim,
@@ -369,6 +540,8 @@ int check_layer(const zg_lm_layer& d, size_t i) {
     ZG_REQUIRE(d.ff == ZG_LM_FF_NONE || d.ff_width >= 1, ZG_ERR_ARG, "layer %zu: feed-forward width %d", i, d.ff_width);
     ZG_REQUIRE(d.ff != ZG_LM_FF_MOE || (d.experts >= 1 && d.experts <= 256 && d.top >= 1 && d.top <= d.experts), ZG_ERR_UNSUPPORTED,
                "layer %zu: %d experts, %d chosen (at most 256 experts)", i, d.experts, d.top);
+    ZG_REQUIRE((d.ff_act == ZG_LM_ACT_GLU_SILU || d.ff_act == ZG_LM_ACT_GELU) && (d.router == ZG_LM_ROUTE_SOFTMAX_ALL || d.router == ZG_LM_ROUTE_TOP_LOGITS),
+               ZG_ERR_ARG, "layer %zu: expert activation %d, router rule %d", i, d.ff_act, d.router);
     return ZG_OK;
 }
 
@@ -380,32 +553,101 @@ int enqueue_layers(zg_lm* g, int M, int n_ent, bool capturing, bool single) {
     const int W = g->W, MS = g->MS, NS = g->NS;
     const int *d_ids = g->meta, *d_pos = d_ids + MS, *d_slot = d_pos + MS, *d_prev = d_slot + MS, *d_last = d_prev + MS, *d_want = d_last + MS;
     const int *d_estart = d_want + MS, *d_elen = d_estart + NS, *d_eslot = d_elen + NS;
+    const int* d_off = g->meta + meta_row_off(g);
     const bool f32 = g->f32;
     const float eps = g->cfg.norm_eps;
     const bool few = M <= kGemvMaxRows;
-    ZG_TRY(launch_embed(g->embed, d_ids, g->x, M, W, g->V, g->flag, s));
+    const bool canon = g->canon >= 1;
+    const bool readd = (g->cfg.flags & ZG_LM_LOOP_READD) && g->cfg.loop_times > 1;
+    ZG_TRY(launch_embed(g->embed, d_ids, g->x, readd ? g->x0 : nullptr, g->embed_scale, M, W, g->V, g->flag, s));
+    // h + conv(h) of a sublayer's input, and the tail of the slots moved on
+    auto input_conv = [&](const float* w, size_t off) -> int {
+        ConvArgs c;
+        c.in = g->h; c.ld_in = W; c.out = g->hc; c.ld_out = W; c.C = W; c.taps = g->canon; c.w = w; c.flags = CONV_RESIDUAL;
+        c.tail = g->seq_state + off; c.slot_stride = g->seq_floats;
+        return launch_causal_conv(c, M, n_ent, d_off, d_slot, d_estart, d_elen, d_eslot, s);
+    };
     bool h_ready = false;  // g->h already holds this pass's shifted norm (written by the previous pass's fused tail)
     for (int p = 0; p < g->n_passes; ++p) {
         const Pass& ps = g->passes[p];
         const LayerW& L = g->layers[ps.layer];
         const zg_lm_layer& d = L.d;
         const int H = d.heads, D = d.dim, Vd = d.vdim;
+        if (ps.readd) ZG_TRY(launch_add_rows(g->x, g->x0, M, W, s));
         if (!h_ready)
-            ZG_TRY(launch_norm_shift(g->x, L.norm1, L.shift, eps, g->h, M, W, d_prev, d_slot, g->shift_state + (size_t)p * W,
-                                     (size_t)g->n_passes * W, d_last, g->last_h + (size_t)p * NS * W, s));
+            ZG_TRY(launch_norm_shift(g->x, L.norm1, canon ? nullptr : L.shift, eps, g->h, M, W, d_prev, d_slot, g->shift_state + (size_t)p * W,
+                                     (size_t)g->n_passes * W, canon ? nullptr : d_last, g->last_h + (size_t)p * NS * W, s));
         h_ready = false;
+        const float* hin = g->h;  // what the sublayer reads
+        if (canon) {
+            ZG_TRY(input_conv(L.canon1, ps.canon1_off));
+            hin = g->hc;
+        }
         // one row per entry: the pass's last sum is fused with the next pass's norm + shift (tail below)
         auto tail = [&](const float* y, const float* yexp, const float* weight, int top, const float* wb) -> int {
-            if (!single || p + 1 >= g->n_passes) return ZG_OK;
+            if (!single || p + 1 >= g->n_passes || canon) return ZG_OK;
             const LayerW& N = g->layers[g->passes[p + 1].layer];
             return launch_sum_norm_shift(g->x, y, yexp, weight, top, wb, N.norm1, N.shift, eps, g->h, M, W, d_slot, g->shift_state + (size_t)(p + 1) * W,
                                          (size_t)g->n_passes * W, d_last, g->last_h + (size_t)(p + 1) * NS * W, s, &h_ready);
         };
         Linear lin;
-        if (d.mixer == ZG_LM_MIX_HGRN2) {
+        if (d.mixer == ZG_LM_MIX_PARALLEL) {
+            const int G = d.kv_heads, C = d.lru_width, NB = d.lru_blocks, BS = C / NB, HV = H * Vd, NP = L.n_cat;
+            const int oy = H * D + G * D + G * Vd, ox = oy + C;  // columns of the two branches of the recurrent unit
+            const Rotary rot{L.rot_freq, d.rot_dims, 1.0f};
+            lin = Linear();
+            lin.A = hin; lin.lda = W; lin.B = L.wcat; lin.ldb = W; lin.C = g->proj; lin.ldc = NP; lin.M = M; lin.N = NP; lin.K = W;
+            ZG_TRY(launch_linear(lin, f32, s));
+            // left: attention inside the window
+            ZG_TRY(launch_window_prep(g->proj, NP, M, H, G, D, Vd, rot, L.vfreq, d_pos, d_slot, g->page_table, g->max_pages, g->P, ps.cache, s));
+            ZG_TRY(launch_window_attention(g->proj, NP, g->o, HV, M, H, G, D, Vd, d.scale, d.window, L.sink, L.talk, L.vfreq, d_pos, d_slot,
+                                           g->page_table, g->max_pages, g->P, ps.cache, s));
+            lin = Linear();
+            lin.A = g->o; lin.lda = HV; lin.B = L.o; lin.ldb = HV; lin.C = g->y; lin.ldc = W; lin.M = M; lin.N = W; lin.K = HV;
+            ZG_TRY(launch_linear(lin, f32, s));
+            // right: convolution, gates block by block, the recurrence
+            ConvArgs cv;
+            cv.in = g->proj + ox; cv.ld_in = NP; cv.out = g->ta; cv.ld_out = C; cv.C = C; cv.taps = d.lru_conv; cv.w = L.convw; cv.bias = L.convb;
+            cv.pre_bias = L.xb; cv.tail = g->seq_state + ps.conv_off; cv.slot_stride = g->seq_floats;
+            ZG_TRY(launch_causal_conv(cv, M, n_ent, d_off, d_slot, d_estart, d_elen, d_eslot, s));
+            for (int which = 0; which < 2; ++which) {
+                lin = Linear();
+                lin.A = g->ta; lin.lda = C; lin.a_zoff = BS; lin.B = which ? L.ri : L.ra; lin.ldb = BS; lin.b_zoff = (long long)BS * BS;
+                lin.C = which ? g->tc : g->tb; lin.ldc = C; lin.c_zoff = BS; lin.M = M; lin.N = BS; lin.K = BS; lin.nz = NB;
+                ZG_TRY(launch_linear(lin, f32, s));
+            }
+            ZG_TRY(launch_rglru_scan(g->ta, C, g->tb, g->tc, C, L.rab, L.rib, L.lam, g->proj + oy, NP, L.yb, g->td, C, C, g->seq_state + ps.rec_off,
+                                     g->seq_floats, d_estart, d_elen, d_eslot, n_ent, s));
+            lin = Linear();
+            lin.A = g->td; lin.lda = C; lin.B = L.ro; lin.ldb = C; lin.C = g->y2; lin.ldc = W; lin.M = M; lin.N = W; lin.K = C;
+            ZG_TRY(launch_linear(lin, f32, s));
+            ZG_TRY(launch_pair_norm_mean(g->y, g->y2, L.left_out, L.right_out, eps, g->y, M, W, s));
+        } else if (d.mixer == ZG_LM_MIX_CHANNEL_DELTA) {
+            const int G = d.kv_heads, HV = H * Vd, CC = 2 * G * D + HV, RA = d.decay_rank, RG = d.gate_rank, NP = L.n_cat;
+            lin = Linear();
+            lin.A = hin; lin.lda = W; lin.B = L.wcat; lin.ldb = W; lin.C = g->proj; lin.ldc = NP; lin.M = M; lin.N = NP; lin.K = W;
+            ZG_TRY(launch_linear(lin, f32, s));
+            ConvArgs cv;
+            cv.in = g->proj; cv.ld_in = NP; cv.out = g->ta; cv.ld_out = CC; cv.C = CC; cv.taps = d.conv; cv.w = L.convw; cv.flags = CONV_SILU;
+            cv.tail = g->seq_state + ps.conv_off; cv.slot_stride = g->seq_floats;
+            ZG_TRY(launch_causal_conv(cv, M, n_ent, d_off, d_slot, d_estart, d_elen, d_eslot, s));
+            lin = Linear();  // the decay's second step
+            lin.A = g->proj + CC + H; lin.lda = NP; lin.B = L.a2; lin.ldb = RA; lin.C = g->tb; lin.ldc = H * D; lin.M = M; lin.N = H * D; lin.K = RA;
+            ZG_TRY(launch_linear(lin, f32, s));
+            lin = Linear();  // the output gate's second step
+            lin.A = g->proj + CC + H + RA; lin.lda = NP; lin.B = L.g2; lin.ldb = RG; lin.C = g->tc; lin.ldc = HV; lin.M = M; lin.N = HV; lin.K = RG;
+            ZG_TRY(launch_linear(lin, f32, s));
+            ZG_TRY(launch_delta_prep(g->ta, CC, G, D, g->proj + CC, NP, H, g->tb, H * D, L.a_log, L.dt_bias, M, s));
+            ZG_TRY(launch_delta_scan(g->ta, CC, g->ta + 2 * G * D, CC, g->proj + CC, NP, g->tb, H * D, g->td, HV, H, G, D, Vd,
+                                     g->seq_state + ps.rec_off, g->seq_floats, d_estart, d_elen, d_eslot, n_ent, s));
+            ZG_TRY(launch_norm_gate(g->td, HV, H, Vd, M, L.hnorm, eps, g->tc, HV, s));
+            lin = Linear();
+            lin.A = g->td; lin.lda = HV; lin.B = L.o; lin.ldb = HV; lin.C = g->y; lin.ldc = W; lin.M = M; lin.N = W; lin.K = HV;
+            ZG_TRY(launch_linear(lin, f32, s));
+        } else if (d.mixer == ZG_LM_MIX_HGRN2) {
             const int HD = H * D, HV = H * Vd, NP = 2 * HD + HV;
             lin = Linear();
-            lin.A = g->h; lin.lda = W; lin.B = L.qfv; lin.ldb = W; lin.C = g->proj; lin.ldc = NP; lin.M = M; lin.N = NP; lin.K = W;
+            lin.A = hin; lin.lda = W; lin.B = L.qfv; lin.ldb = W; lin.C = g->proj; lin.ldc = NP; lin.M = M; lin.N = NP; lin.K = W;
             ZG_TRY(launch_linear(lin, f32, s));
             ZG_TRY(launch_hgrn2_scan(g->proj, NP, g->o, HV, g->hgrn_state + ps.hgrn_off, g->hgrn_floats, d_estart, d_elen, d_eslot, n_ent, M, H, D, Vd,
                                      L.fb, L.lower, g->scan_ws, g->scan_ws_floats, s));
@@ -417,7 +659,7 @@ int enqueue_layers(zg_lm* g, int M, int n_ent, bool capturing, bool single) {
             const int R = d.rot_dim, KR = d.kv_rank, QR = d.q_rank, HV = H * Vd, NP = QR + KR + R;
             const Rotary rot{L.rot_freq, d.rot_dims, L.rot_amp};
             lin = Linear();
-            lin.A = g->h; lin.lda = W; lin.B = L.dqkv; lin.ldb = W; lin.C = g->proj; lin.ldc = NP; lin.M = M; lin.N = NP; lin.K = W;
+            lin.A = hin; lin.lda = W; lin.B = L.dqkv; lin.ldb = W; lin.C = g->proj; lin.ldc = NP; lin.M = M; lin.N = NP; lin.K = W;
             ZG_TRY(launch_linear(lin, f32, s));
             ZG_TRY(launch_latent_prep(g->proj, NP, M, QR, KR, R, L.dq_norm, L.dkv_norm, eps, rot, d_pos, d_slot, g->page_table, g->max_pages, g->P,
                                       g->cq, ps.cache, s));
@@ -450,9 +692,14 @@ int enqueue_layers(zg_lm* g, int M, int n_ent, bool capturing, bool single) {
             if (!h_ready) ZG_TRY(launch_norm_add(g->x, g->y, L.norm1b, eps, M, W, s));
         }
         const int F = d.ff_width;
+        hin = g->h;
+        if (canon && d.ff != ZG_LM_FF_NONE) {
+            ZG_TRY(input_conv(L.canon2, ps.canon2_off));
+            hin = g->hc;
+        }
         if (d.ff == ZG_LM_FF_DENSE) {
             lin = Linear();
-            lin.A = g->h; lin.lda = W; lin.B = L.up; lin.ldb = W; lin.C = g->u; lin.ldc = F; lin.M = M; lin.N = F; lin.K = W; lin.act = ACT_RELU2;
+            lin.A = hin; lin.lda = W; lin.B = L.up; lin.ldb = W; lin.C = g->u; lin.ldc = F; lin.M = M; lin.N = F; lin.K = W; lin.act = ACT_RELU2;
             ZG_TRY(launch_linear(lin, f32, s));
             lin = Linear();
             lin.A = g->u; lin.lda = F; lin.B = L.down; lin.ldb = F; lin.C = g->y; lin.ldc = W; lin.M = M; lin.N = W; lin.K = F;
@@ -461,20 +708,25 @@ int enqueue_layers(zg_lm* g, int M, int n_ent, bool capturing, bool single) {
             if (!h_ready) ZG_TRY(launch_norm_add(g->x, g->y, L.norm2b, eps, M, W, s));
         } else if (d.ff == ZG_LM_FF_MOE) {
             const int E = d.experts, top = d.top, NA = M * top;
-            ZG_TRY(launch_route(g->h, M, W, L.router, L.correction, E, top, g->pick, g->wt, s));
+            const bool glu = d.ff_act == ZG_LM_ACT_GLU_SILU;
+            const int UF = glu ? 2 * F : F;
+            ZG_TRY(launch_route(hin, M, W, L.router, L.correction, E, top, g->pick, g->wt, d.router == ZG_LM_ROUTE_TOP_LOGITS, s));
             Linear up, dn;
-            up.A = g->h; up.lda = W; up.a_div = top; up.B = L.gu; up.ldb = W; up.b_zoff = (long long)2 * F * W; up.C = g->gu_buf; up.ldc = 2 * F;
-            up.N = 2 * F; up.K = W;
+            up.A = hin; up.lda = W; up.a_div = top; up.B = L.gu; up.ldb = W; up.b_zoff = (long long)UF * W; up.C = g->gu_buf; up.ldc = UF;
+            up.N = UF; up.K = W;
+            if (!glu) up.act = ACT_GELU_ERF;
             dn.A = g->hb; dn.lda = F; dn.B = L.edown; dn.ldb = F; dn.b_zoff = (long long)W * F; dn.C = g->ye; dn.ldc = W; dn.N = W; dn.K = F;
             if (few) {  // one batch per assignment, its expert's matrices looked up on the device
                 up.M = dn.M = 1; up.nz = dn.nz = NA; up.z_group = dn.z_group = g->pick;
-                up.c_zoff = 2 * F; dn.c_zoff = W;
+                up.c_zoff = UF; dn.c_zoff = W;
             } else {  // assignments sorted by expert, grouped products
                 ZG_TRY(launch_group(g->pick, NA, E, g->grp_off, g->sorted, g->inv, s));
                 up.M = dn.M = NA; up.a_rows = g->sorted; up.grp_off = dn.grp_off = g->grp_off; up.n_groups = dn.n_groups = E;
             }
             ZG_TRY(launch_linear(up, f32, s));
-            if (few) {  // the gated activation is applied where the second product reads its rows
+            if (!glu) {  // the first product's epilogue has applied the activation
+                dn.A = g->gu_buf; dn.lda = F;
+            } else if (few) {  // the gated activation is applied where the second product reads its rows
                 dn.A = g->gu_buf; dn.lda = 2 * F; dn.a_glu = F;
             } else {
                 ZG_TRY(launch_glu(g->gu_buf, g->hb, NA, F, s));
@@ -489,7 +741,7 @@ int enqueue_layers(zg_lm* g, int M, int n_ent, bool capturing, bool single) {
         }
     }
     // the rows the last tokens of the entries left for the token shift of their successors
-    ZG_TRY(launch_commit_rows(g->shift_state, (size_t)g->n_passes * W, g->last_h, W, d_eslot, n_ent, W, g->n_passes, W, (size_t)NS * W, s));
+    if (!canon) ZG_TRY(launch_commit_rows(g->shift_state, (size_t)g->n_passes * W, g->last_h, W, d_eslot, n_ent, W, g->n_passes, W, (size_t)NS * W, s));
 
     return ZG_OK;
 }
@@ -504,6 +756,7 @@ int run_portion(zg_lm* g, const std::vector<Piece>& pieces, float* logits_out, c
     const int n_ent = (int)pieces.size();
     int *ids = g->h_meta, *pos = ids + MS, *slot = pos + MS, *prev = slot + MS, *lastent = prev + MS, *want_rows = lastent + MS;
     int *ent_start = want_rows + MS, *ent_len = ent_start + NS, *ent_slot = ent_len + NS;
+    int* row_off = g->h_meta + meta_row_off(g);
     std::vector<std::pair<int, size_t>> wants;  // (row of the portion, output row)
     int r = 0;
     for (int e = 0; e < n_ent; ++e) {
@@ -517,6 +770,7 @@ int run_portion(zg_lm* g, const std::vector<Piece>& pieces, float* logits_out, c
             slot[r] = pc.slot;
             prev[r] = t > 0 ? r - 1 : -1;
             lastent[r] = t == pc.n - 1 ? e : -1;
+            row_off[r] = t;
         }
         for (auto& w : pc.wants) wants.push_back({ent_start[e] + w.first, w.second});
         const Slot& sl = g->slots[pc.slot];
@@ -665,6 +919,17 @@ int step_impl(zg_lm* g, const zg_lm_entry* entries, size_t n_entries, float* log
         out_base += e.n_want;
     }
     if (!pieces.empty()) ZG_TRY(run_portion(g, pieces, logits_out, sampler));
+    if (g->keep_tokens > 0)  // pages whose every token lies behind the longest window return to the pool
+        for (size_t i = 0; i < n_entries; ++i) {
+            Slot& sl = g->slots[entries[i].seq];
+            if (sl.len + 1 <= (size_t)g->keep_tokens) continue;
+            const size_t dead = (sl.len + 1 - g->keep_tokens) / g->P;  // the next token sees positions >= len + 1 - keep
+            for (size_t pg = 0; pg < dead && pg < sl.pages.size(); ++pg)
+                if (sl.pages[pg] >= 0) {
+                    g->free_pages.push_back(sl.pages[pg]);
+                    sl.pages[pg] = -1;
+                }
+        }
     return ZG_OK;
 }
 
@@ -699,6 +964,8 @@ int zg_lm_create(zg_lm** out, const zg_lm_config* config, int device) {
     g->max_pages = (int)((max_tokens + g->P - 1) / g->P);
     g->n_pages = g->max_pages + g->NS;  // every open sequence may leave one page partly used
     g->logit_rows = std::min(g->MS, 256);
+    g->canon = config->canon_taps;
+    g->embed_scale = config->embed_scale != 0.0f ? config->embed_scale : 1.0f;
     int status = ZG_OK;
     for (size_t i = 0; i < config->n_layers && status == ZG_OK; ++i) {
         status = check_layer(config->layers[i], i);
@@ -707,6 +974,10 @@ int zg_lm_create(zg_lm** out, const zg_lm_config* config, int device) {
         g->layers.push_back(L);
     }
     g->cfg.layers = nullptr;
+    if (status == ZG_OK && (g->canon < 0 || g->canon > 16)) {
+        set_error("lm_create: %d taps of the input convolution (0 to 16)", g->canon);
+        status = ZG_ERR_ARG;
+    }
     const int n = (int)config->n_layers;
     int a = 0, b = 0, k = 1;
     if (status == ZG_OK && config->loop_times > 1) {
@@ -727,9 +998,23 @@ int zg_lm_create(zg_lm** out, const zg_lm_config* config, int device) {
     };
     for (int i = 0; i < a; ++i) add(i);
     for (int t = 0; t < k; ++t)
-        for (int i = a; i < b; ++i) add(i);
+        for (int i = a; i < b; ++i) {
+            add(i);
+            g->passes.back().readd = t > 0 && i == a && (config->flags & ZG_LM_LOOP_READD);
+        }
     for (int i = (k > 1 ? b : 0); i < n; ++i) add(i);
     g->n_passes = (int)g->passes.size();
+    // how far back any attention pass looks: pages behind that are given back while a sequence is still open
+    bool attends = false, bounded = true;
+    for (const Pass& ps : g->passes) {
+        const zg_lm_layer& d = g->layers[ps.layer].d;
+        if (d.mixer == ZG_LM_MIX_LATENT_ATTENTION || (d.mixer == ZG_LM_MIX_PARALLEL && d.window == 0)) attends = true, bounded = false;
+        if (d.mixer == ZG_LM_MIX_PARALLEL && d.window > 0) {
+            attends = true;
+            g->keep_tokens = std::max(g->keep_tokens, d.window);
+        }
+    }
+    if (!attends || !bounded) g->keep_tokens = 0;
     Bump measure{nullptr};
     layout(g, measure);
     g->arena_bytes = measure.off + 256;
@@ -764,11 +1049,21 @@ int zg_lm_create(zg_lm** out, const zg_lm_config* config, int device) {
     zero_kernel<<<1, 256, 0, g->stream>>>(reinterpret_cast<float*>(g->flag), 16);
     zero_kernel<<<(unsigned)(((size_t)g->NS * g->max_pages + 255) / 256), 256, 0, g->stream>>>(reinterpret_cast<float*>(g->page_table),
                                                                                             (size_t)g->NS * g->max_pages);
+    if (g->seq_floats) {
+        const size_t nsq = (size_t)g->NS * g->seq_floats;
+        zero_kernel<<<(unsigned)((nsq + 255) / 256), 256, 0, g->stream>>>(g->seq_state, nsq);
+    }
     for (LayerW& L : g->layers)
-        if (L.d.mixer == ZG_LM_MIX_LATENT_ATTENTION) {
+        if (L.d.mixer == ZG_LM_MIX_LATENT_ATTENTION || L.d.mixer == ZG_LM_MIX_PARALLEL) {
             std::vector<float> freq;
             rotary_table(L.d, freq, L.rot_amp);
             ZG_LM_TRY_HIP(hipMemcpy(L.rot_freq, freq.data(), std::max<size_t>(1, L.d.rot_dims / 2) * sizeof(float), hipMemcpyHostToDevice));
+            if (L.d.mixer == ZG_LM_MIX_PARALLEL) {  // the values turn at the unscaled frequencies of their own size
+                const int vd = L.d.vdim;
+                std::vector<float> vf(std::max(1, vd / 2));
+                for (int i = 0; i < vd / 2; ++i) vf[i] = (float)pow((double)L.d.rot_base, -2.0 * i / vd);
+                ZG_LM_TRY_HIP(hipMemcpy(L.vfreq, vf.data(), vf.size() * sizeof(float), hipMemcpyHostToDevice));
+            }
         }
     ZG_LM_TRY_HIP(hipStreamSynchronize(g->stream));
 #undef ZG_LM_TRY_HIP
@@ -876,6 +1171,10 @@ int zg_lm_seq_open(zg_lm* g, int* seq_out) {
         zero_kernel<<<(unsigned)((g->hgrn_floats + 255) / 256), 256, 0, g->stream>>>(g->hgrn_state + (size_t)sidx * g->hgrn_floats, g->hgrn_floats);
         ZG_HIP(hipGetLastError());
     }
+    if (g->seq_floats) {
+        zero_kernel<<<(unsigned)((g->seq_floats + 255) / 256), 256, 0, g->stream>>>(g->seq_state + (size_t)sidx * g->seq_floats, g->seq_floats);
+        ZG_HIP(hipGetLastError());
+    }
     Slot& sl = g->slots[sidx];
     sl.open = true;
     sl.len = 0;
@@ -887,7 +1186,8 @@ int zg_lm_seq_open(zg_lm* g, int* seq_out) {
 int zg_lm_seq_close(zg_lm* g, int seq) {
     ZG_REQUIRE(g && seq >= 0 && seq < g->NS && g->slots[seq].open, ZG_ERR_ARG, "lm_seq_close: sequence %d is not open", seq);
     Slot& sl = g->slots[seq];
-    for (int p : sl.pages) g->free_pages.push_back(p);
+    for (int p : sl.pages)
+        if (p >= 0) g->free_pages.push_back(p);
     sl.pages.clear();
     sl.open = false;
     sl.len = 0;

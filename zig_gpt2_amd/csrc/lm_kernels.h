@@ -15,7 +15,7 @@ namespace zg {
 namespace lm {
 
 // ------------------------------------------------------------------------------------------------ linear maps
-enum { ACT_NONE = 0, ACT_RELU2 = 1 };
+enum { ACT_NONE = 0, ACT_RELU2 = 1, ACT_GELU_ERF = 2 };
 
 // C[m][n] = act( sum_k A[arow(m)][k] * B[n][k] )      for m < M, n < N
 //   arow(m) = a_rows ? a_rows[m] / a_div : m          (row gather: a token's row feeds each of its expert assignments)
@@ -34,6 +34,7 @@ struct Linear {
     int ldc = 0;
     int M = 0, N = 0, K = 0;
     int act = ACT_NONE;
+    const float* bias = nullptr;  // [N], added before the activation (one vector for every batch: not with nz > 1 or groups)
     int a_glu = 0;  // > 0 (row-vector kernel only): A rows are [gate (a_glu) | up (a_glu)] and enter as silu(gate) * up, K = a_glu
     int nz = 1;
     long long a_zoff = 0, b_zoff = 0, c_zoff = 0;
@@ -47,7 +48,8 @@ constexpr int kGemvMaxRows = 8;
 
 // ------------------------------------------------------------------------------------------------ norms, embedding, shift
 // x[m] = table[ids[m]] (bf16 -> fp32); an id outside [0, vocab) raises *flag (pinned or device int) and yields a zero row.
-int launch_embed(const bf16_t* table, const int* ids, float* x, int M, int W, int vocab, int* flag, hipStream_t s);
+// scale multiplies the row; x_copy (may be null) receives the same rows.
+int launch_embed(const bf16_t* table, const int* ids, float* x, float* x_copy, float scale, int M, int W, int vocab, int* flag, hipStream_t s);
 // RMS norm with a weight stored as an offset from one, then the token shift:
 //   h[m] = x[m] / rms(x[m]) * (1 + w);   out[m] = h[m] + (h[prev(m)] - h[m]) * mu
 // prev(m) = row_prev[m] when >= 0, else the row kept for the slot: shift_state[row_slot[m]] (zeros for a new sequence).
@@ -111,10 +113,68 @@ int launch_latent_attention_tiles(const float* qa, float* ctx, int M, int H, int
                                   const int* ent_slot, int n_entries, const int* row_pos, const int* page_table, int max_pages, int page_tokens,
                                   const float* cache, hipStream_t s, bool* taken);
 
+// ------------------------------------------------------------------------------------------------ causal convolutions with a tail
+// out[m][c] = act( bias[c] + sum_j w[c][j] * in(m - (taps - 1) + j)[c]  (+ in(m)[c] with CONV_RESIDUAL) ),  in(.) = in[.] + pre_bias;
+// inputs in front of the step come from the slot's tail ([taps - 1][C] floats at tail + slot * slot_stride, oldest first; zeros
+// for a new sequence), which a second launch then moves on by the entry's tokens.  row_off[m]: place of row m inside its entry.
+enum { CONV_RESIDUAL = 1, CONV_SILU = 2 };
+struct ConvArgs {
+    const float* in = nullptr;
+    int ld_in = 0;
+    float* out = nullptr;
+    int ld_out = 0;
+    int C = 0, taps = 1;
+    const float* w = nullptr;         // [C][taps] fp32, last column = the current token
+    const float* bias = nullptr;      // [C] or null
+    const float* pre_bias = nullptr;  // [C] or null: a bias of the input rows (the tail holds inputs with it)
+    int flags = 0;
+    float* tail = nullptr;
+    size_t slot_stride = 0;
+};
+int launch_causal_conv(const ConvArgs& a, int M, int n_entries, const int* row_off, const int* row_slot, const int* ent_start, const int* ent_len,
+                       const int* ent_slot, hipStream_t s);
+// x[m] += y[m]
+int launch_add_rows(float* x, const float* y, int M, int W, hipStream_t s);
+
+// ------------------------------------------------------------------------------------------------ windowed attention (sink, mixed heads, rotated values)
+// proj rows [q (H D) | k (G D) | v (G V)]: q rotated in place; the rotated key and the value rotated over all V channels (pair i by
+// pos * vfreq[i]) written to the token's cache row [G D | G V] (cache row of (slot, pos) through the page table).
+int launch_window_prep(float* proj, int ld, int M, int H, int G, int D, int V, Rotary rot, const float* vfreq, const int* row_pos,
+                       const int* row_slot, const int* page_table, int max_pages, int page_tokens, float* cache, hipStream_t s);
+// out[m][h] = turn_back_pos( sum_j w_h(j) value_(h / (H/G))(j) ),  w_h = sum_g talk[h][g] p_g,
+// p_g(j) = exp(s_g(j)) / (exp(sink_g) + sum_j' exp(s_g(j'))),  s_g(j) = scale q_g . k(j),  over the keys pos - window < j <= pos
+// (window 0: all j <= pos).  sink / talk may be null (no sink / no mix).
+int launch_window_attention(const float* q, int ldq, float* out, int ldo, int M, int H, int G, int D, int V, float scale, int window,
+                            const float* sink, const float* talk, const float* vfreq, const int* row_pos, const int* row_slot,
+                            const int* page_table, int max_pages, int page_tokens, const float* cache, hipStream_t s);
+
+// ------------------------------------------------------------------------------------------------ real-gated linear recurrent unit
+// Per entry and channel c: r = sigmoid(gr + br), i = sigmoid(gi + bi), a = exp(-8 r softplus(lam)), S = a S + sqrt(1 - a^2) i u,
+// out = S * gelu_tanh(y + by); S = state[slot][c], read at the start of the entry and written back at its end.
+int launch_rglru_scan(const float* u, int ldu, const float* gr, const float* gi, int ldg, const float* br, const float* bi, const float* lam,
+                      const float* y, int ldy, const float* by, float* out, int ldo, int C, float* state, size_t slot_stride, const int* ent_start,
+                      const int* ent_len, const int* ent_slot, int n_entries, hipStream_t s);
+// y[m] = (l[m] / rms(l[m]) * wl + r[m] / rms(r[m]) * wr) / 2
+int launch_pair_norm_mean(const float* l, const float* r, const float* wl, const float* wr, float eps, float* y, int M, int W, hipStream_t s);
+
+// ------------------------------------------------------------------------------------------------ gated delta rule, decay per key channel
+// In place: the G query heads and G key heads of qk rows ([q (G D) | k (G D)]) to unit length (q also times D^-1/2);
+// beta <- sigmoid(beta);  dec[h][d] <- exp(-exp(a_log[h]) * softplus(dec[h][d] + dt_bias[h][d])).
+int launch_delta_prep(float* qk, int ldqk, int G, int D, float* beta, int ldb, int H, float* dec, int ldd, const float* a_log,
+                      const float* dt_bias, int M, hipStream_t s);
+// Per entry and head h (query / key head h / (H / G)), token by token on S = state[slot][h] ([D][V] fp32):
+//   S <- diag(dec) S;  u = beta (v - S^T k);  S <- S + k u^T;  out = S^T q.
+int launch_delta_scan(const float* qk, int ldqk, const float* v, int ldv, const float* beta, int ldb, const float* dec, int ldd, float* out,
+                      int ldo, int H, int G, int D, int V, float* state, size_t slot_stride, const int* ent_start, const int* ent_len,
+                      const int* ent_slot, int n_entries, hipStream_t s);
+// In place over M * rows_per_m vectors of `width` floats: v / rms(v) * w * sigmoid(gate) (gate laid out like v, row stride ldg)
+int launch_norm_gate(float* v, int ld, int rows_per_m, int width, int M, const float* w, float eps, const float* gate, int ldg, hipStream_t s);
+
 // ------------------------------------------------------------------------------------------------ mixture of experts
 // Per row: z = router . g (fp32), s = softmax(z), the `top` experts by s + correction (lowest index wins a tie), weights s.
+// top_logits: z += correction (a bias), the `top` largest z (lowest index wins a tie), weights = softmax over the chosen z.
 int launch_route(const float* g, int M, int W, const bf16_t* router, const float* correction, int E, int top, int* pick, float* weight,
-                 hipStream_t s);
+                 bool top_logits, hipStream_t s);
 // Sort the M * top assignments by expert: grp_off[E + 1], sorted[p] = assignment at sorted position p, inv[a] = position of a.
 int launch_group(const int* pick, int n_assign, int E, int* grp_off, int* sorted, int* inv, hipStream_t s);
 // h[p][j] = silu(gu[p][j]) * gu[p][F + j]

@@ -35,12 +35,17 @@ __device__ __forceinline__ float row_inv_rms(const float* v, int n, float eps, f
 __device__ __forceinline__ float silu_f(float z) { return z / (1.0f + expf(-z)); }
 __device__ __forceinline__ float sigmoid_f(float z) { return 1.0f / (1.0f + expf(-z)); }
 
-__global__ __launch_bounds__(256) void embed_kernel(const bf16_t* table, const int* ids, float* x, int W, int vocab, int* flag) {
+__global__ __launch_bounds__(256) void embed_kernel(const bf16_t* table, const int* ids, float* x, float* x_copy, float scale, int W, int vocab,
+                                                    int* flag) {
     const int m = blockIdx.x, id = ids[m];
     const bool ok = id >= 0 && id < vocab;
     if (!ok && threadIdx.x == 0) *flag = 1;
     const bf16_t* row = table + (size_t)(ok ? id : 0) * W;
-    for (int i = threadIdx.x; i < W; i += blockDim.x) x[(size_t)m * W + i] = ok ? __uint_as_float((uint32_t)row[i] << 16) : 0.0f;
+    for (int i = threadIdx.x; i < W; i += blockDim.x) {
+        const float v = ok ? __uint_as_float((uint32_t)row[i] << 16) * scale : 0.0f;
+        x[(size_t)m * W + i] = v;
+        if (x_copy) x_copy[(size_t)m * W + i] = v;
+    }
 }
 
 // Rows of up to 256 * kRowRegs floats are held in registers between the statistics and the result: every operand is requested
@@ -816,9 +821,9 @@ __global__ __launch_bounds__(256) void row_argmax_kernel(const float* logits, in
 
 }  // namespace
 
-int launch_embed(const bf16_t* table, const int* ids, float* x, int M, int W, int vocab, int* flag, hipStream_t s) {
+int launch_embed(const bf16_t* table, const int* ids, float* x, float* x_copy, float scale, int M, int W, int vocab, int* flag, hipStream_t s) {
     if (M <= 0) return ZG_OK;
-    embed_kernel<<<M, 256, 0, s>>>(table, ids, x, W, vocab, flag);
+    embed_kernel<<<M, 256, 0, s>>>(table, ids, x, x_copy, scale, W, vocab, flag);
     ZG_HIP(hipGetLastError());
     return ZG_OK;
 }

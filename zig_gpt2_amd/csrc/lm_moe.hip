@@ -26,8 +26,10 @@ __device__ __forceinline__ float block_allsum(float v, float* s_red) {
 // One workgroup per row.  The four waves share the experts (wave w scores experts w, w + 4, ...): a router row is one dot
 // product, the lanes take 16-byte pieces of it and every piece of up to 2048 channels is requested before the first is used; the
 // logits meet in the LDS and wave 0 does the softmax and the choice, lane e % 64 holding expert e (four slots per lane).
+// top_logits: the correction is a bias of the logits, the largest logits are chosen and the weights are the softmax over the chosen
+// logits alone.
 __global__ __launch_bounds__(256) void route_kernel(const float* g, int M, int W, const bf16_t* router, const float* correction, int E, int top,
-                                                    int* pick, float* weight) {
+                                                    int* pick, float* weight, int top_logits) {
     __shared__ float s_z[kMaxExperts];
     const int m = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const float* row = g + (size_t)m * W;
@@ -70,6 +72,46 @@ __global__ __launch_bounds__(256) void route_kernel(const float* g, int M, int W
     float z[4], sc[4], ch[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) z[i] = lane + 64 * i < E ? s_z[lane + 64 * i] : -INFINITY;
+    if (top_logits) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) ch[i] = lane + 64 * i < E ? z[i] + correction[lane + 64 * i] : -INFINITY;
+        float ek[4] = {0.0f, 0.0f, 0.0f, 0.0f};  // exp(z_k - z_0) of choice k on lane k % 64, slot k / 64
+        float first = 0.0f;
+        for (int k = 0; k < top; ++k) {
+            float best = -INFINITY;
+            int bi = 0x7fffffff;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (ch[i] > best) {
+                    best = ch[i];
+                    bi = lane + 64 * i;
+                }
+            const float wbest = wave_allmax(best);
+            int cand = (best == wbest) ? bi : 0x7fffffff;
+#pragma unroll
+            for (int off = 1; off < 64; off <<= 1) cand = min(cand, __shfl_xor(cand, off, 64));
+            if (cand == 0x7fffffff) cand = 0;
+            if (k == 0) first = wbest;
+            if ((cand & 63) == lane) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if ((cand >> 6) == i) {
+                        pick[(size_t)m * top + k] = cand;
+                        ch[i] = -INFINITY;
+                    }
+            }
+            if ((k & 63) == lane) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if ((k >> 6) == i) ek[i] = expf(wbest - first);
+            }
+        }
+        const float sum = wave_allsum((ek[0] + ek[1]) + (ek[2] + ek[3]));
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if (lane + 64 * i < top) weight[(size_t)m * top + lane + 64 * i] = ek[i] / sum;
+        return;
+    }
     const float mx = wave_allmax(fmaxf(fmaxf(z[0], z[1]), fmaxf(z[2], z[3])));
     float sum = 0.0f;
 #pragma unroll
@@ -170,11 +212,11 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(float* x, const float*
 }  // namespace
 
 int launch_route(const float* g, int M, int W, const bf16_t* router, const float* correction, int E, int top, int* pick, float* weight,
-                 hipStream_t s) {
+                 bool top_logits, hipStream_t s) {
     if (M <= 0) return ZG_OK;
     ZG_REQUIRE(E >= 1 && E <= kMaxExperts && top >= 1 && top <= E, ZG_ERR_UNSUPPORTED, "router: %d experts, %d chosen (at most %d experts)", E, top,
                kMaxExperts);
-    route_kernel<<<M, 256, 0, s>>>(g, M, W, router, correction, E, top, pick, weight);
+    route_kernel<<<M, 256, 0, s>>>(g, M, W, router, correction, E, top, pick, weight, top_logits ? 1 : 0);
     ZG_HIP(hipGetLastError());
     return ZG_OK;
 }

@@ -1,0 +1,551 @@
+// lm_seq.hip — sequence mixers of the layered-model tier that carry more than a token shift from token to token:
+//   * causal convolutions per channel whose last taps - 1 inputs live in a slot's state (the input convolution of a sublayer,
+//     the short convolutions in front of the recurrences),
+//   * softmax attention inside a sliding window over a paged cache of rotated keys and rotated VALUES, with a sink in the
+//     denominator and the heads' weights mixed by a matrix,
+//   * the real-gated linear recurrent unit (elementwise recurrence),
+//   * the gated delta rule with one decay per key channel (a matrix state per head).
+// Everything here is fp32 in both precision modes: positions, angles, scores, weights, gates, decays, recurrent states.
+#include <math.h>
+
+#include <algorithm>
+
+#include "lm_kernels.h"
+
+namespace zg {
+namespace lm {
+
+namespace {
+
+__device__ __forceinline__ float sigmoid_f(float z) { return 1.0f / (1.0f + expf(-z)); }
+__device__ __forceinline__ float silu_f(float z) { return z / (1.0f + expf(-z)); }
+__device__ __forceinline__ float softplus_f(float z) { return z > 20.0f ? z : log1pf(expf(z)); }
+__device__ __forceinline__ float gelu_tanh_f(float z) { return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z))); }
+
+__device__ __forceinline__ float block_allsum(float v, float* s_red) {
+    v = wave_allsum(v);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+    __syncthreads();
+    if (lane == 0) s_red[wave] = v;
+    __syncthreads();
+    float t = 0.0f;
+    for (int w = 0; w < nw; ++w) t += s_red[w];
+    return t;
+}
+
+// ------------------------------------------------------------------------------------------------ embedding helpers
+__global__ __launch_bounds__(256) void add_rows_kernel(float* x, const float* y, size_t n) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) x[i] += y[i];
+}
+
+// ------------------------------------------------------------------------------------------------ causal convolution
+// Tap j of row m reads the input taps - 1 - j tokens back: a row of the same step when the entry brought that many tokens in
+// front of m, else the slot's tail (the taps - 1 inputs before the step, oldest first; zeros for a new sequence).
+__global__ __launch_bounds__(256) void causal_conv_kernel(const float* in, int ld_in, float* out, int ld_out, int C, int taps, const float* w,
+                                                          const float* bias, const float* pre_bias, int flags, const float* tail,
+                                                          size_t slot_stride, const int* row_off, const int* row_slot) {
+    const int m = blockIdx.x, c = blockIdx.y * blockDim.x + threadIdx.x;
+    if (c >= C) return;
+    const int off = row_off[m], K = taps - 1;
+    const float* tl = tail + (size_t)row_slot[m] * slot_stride;
+    const float pb = pre_bias ? pre_bias[c] : 0.0f;  // a bias of the input itself (the tail holds inputs with it)
+    float acc = bias ? bias[c] : 0.0f;
+    float cur = 0.0f;
+    for (int j = 0; j < taps; ++j) {
+        const int src = off - K + j;
+        const float v = src >= 0 ? in[(size_t)(m - K + j) * ld_in + c] + pb : tl[(size_t)(K + src) * C + c];
+        acc = fmaf(w[(size_t)c * taps + j], v, acc);
+        cur = v;
+    }
+    if (flags & CONV_RESIDUAL) acc += cur;
+    if (flags & CONV_SILU) acc = silu_f(acc);
+    out[(size_t)m * ld_out + c] = acc;
+}
+
+// The new tail of every entry's slot: the last taps - 1 of (old tail, the entry's inputs).  A thread reads all it needs
+// before it writes, and no other thread touches its channel of its slot.
+constexpr int kMaxTaps = 16;
+__global__ __launch_bounds__(256) void conv_tail_kernel(const float* in, int ld_in, int C, int taps, const float* pre_bias, float* tail,
+                                                        size_t slot_stride, const int* ent_start, const int* ent_len, const int* ent_slot) {
+    const int e = blockIdx.x, c = blockIdx.y * blockDim.x + threadIdx.x;
+    if (c >= C) return;
+    const int n = ent_len[e], m0 = ent_start[e], K = taps - 1;
+    if (n <= 0) return;
+    float* tl = tail + (size_t)ent_slot[e] * slot_stride;
+    const float pb = pre_bias ? pre_bias[c] : 0.0f;
+    float val[kMaxTaps];
+#pragma unroll
+    for (int i = 0; i < kMaxTaps; ++i)
+        if (i < K) {
+            const int src = n - K + i;
+            val[i] = src >= 0 ? in[(size_t)(m0 + src) * ld_in + c] + pb : tl[(size_t)(K + src) * C + c];
+        }
+#pragma unroll
+    for (int i = 0; i < kMaxTaps; ++i)
+        if (i < K) tl[(size_t)i * C + c] = val[i];
+}
+
+// ------------------------------------------------------------------------------------------------ windowed attention
+// proj rows: [q (H D) | k (G D) | v (G V)].  q is rotated in place (pairs (2i, 2i + 1) below rot.dims); the rotated key and the
+// value rotated over ALL its channels (pair i by pos * vfreq[i]) go to the token's cache row [G D | G V].
+__global__ __launch_bounds__(256) void window_prep_kernel(float* proj, int ld, int H, int G, int D, int V, Rotary rot, const float* vfreq,
+                                                          const int* row_pos, const int* row_slot, const int* page_table, int max_pages,
+                                                          int page_tokens, float* cache) {
+    const int m = blockIdx.x;
+    const int pos = row_pos[m];
+    const int page = page_table[(size_t)row_slot[m] * max_pages + pos / page_tokens];
+    float* crow = cache + ((size_t)page * page_tokens + pos % page_tokens) * ((size_t)G * (D + V));
+    float* row = proj + (size_t)m * ld;
+    const float fpos = (float)pos;
+    const int half = rot.dims / 2;
+    for (int idx = threadIdx.x; idx < H * half; idx += blockDim.x) {
+        const int h = idx / half, i = idx % half;
+        float* p = row + (size_t)h * D + 2 * i;
+        float sn, cs;
+        sincosf(fpos * rot.freq[i], &sn, &cs);
+        const float a = p[0], b = p[1];
+        p[0] = (a * cs - b * sn) * rot.amp;
+        p[1] = (b * cs + a * sn) * rot.amp;
+    }
+    const float* k = row + (size_t)H * D;
+    for (int idx = threadIdx.x; idx < G * D; idx += blockDim.x) {
+        const int i = idx % D;
+        float out;
+        if (i < rot.dims) {
+            float sn, cs;
+            sincosf(fpos * rot.freq[i >> 1], &sn, &cs);
+            const float own = k[idx], other = k[idx - i + (i ^ 1)];
+            out = ((i & 1) ? own * cs + other * sn : own * cs - other * sn) * rot.amp;
+        } else {
+            out = k[idx];
+        }
+        crow[idx] = out;
+    }
+    const float* v = k + (size_t)G * D;
+    for (int idx = threadIdx.x; idx < G * V; idx += blockDim.x) {
+        const int i = idx % V;
+        float sn, cs;
+        sincosf(fpos * vfreq[i >> 1], &sn, &cs);
+        const float own = v[idx], other = v[idx - i + (i ^ 1)];
+        crow[(size_t)G * D + idx] = (i & 1) ? own * cs + other * sn : own * cs - other * sn;
+    }
+}
+
+// One workgroup per query row, all heads together (the mix of the heads' weights needs every head's weight of a key).
+// Keys are walked in tiles of kWinTile, twice: first the per-head maximum and denominator (with exp(sink) in it), then the
+// normalised weights, their mix over the heads, and the weighted sum of the values of the head's own key/value head.  The
+// result is turned back by the query's position and stored.  Tiles start at the first key of the window: the order of every
+// sum depends on the position alone.
+constexpr int kWinTile = 64;
+constexpr int kWinMaxHeads = 64;
+constexpr int kWinAcc = 16;  // outputs per thread: H * V <= 256 * kWinAcc
+
+__global__ __launch_bounds__(256) void window_attention_kernel(const float* q, int ldq, float* out, int ldo, int H, int G, int D, int V,
+                                                               float scale, int window, const float* sink, const float* talk,
+                                                               const float* vfreq, const int* row_pos, const int* row_slot,
+                                                               const int* page_table, int max_pages, int page_tokens, const float* cache) {
+    extern __shared__ __attribute__((aligned(16))) float s_win[];
+    float* s_q = s_win;                       // [H D]
+    float* s_s = s_q + H * D;                 // [H][kWinTile] scores, then weights
+    float* s_w = s_s + H * kWinTile;          // [H][kWinTile] mixed weights
+    float* s_talk = s_w + H * kWinTile;       // [H H]
+    float* s_o = s_talk + H * H;              // [H V]
+    __shared__ float s_max[kWinMaxHeads], s_den[kWinMaxHeads];
+    __shared__ int s_row[kWinTile];  // cache row of every key of the tile
+    const int m = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int pos = row_pos[m];
+    const int* pages = page_table + (size_t)row_slot[m] * max_pages;
+    const int j_lo = window > 0 ? max(0, pos - window + 1) : 0;
+    const int n_keys = pos - j_lo + 1;
+    const int rep = H / G;
+    const size_t cstride = (size_t)G * (D + V);
+    for (int i = tid; i < H * D; i += blockDim.x) s_q[i] = q[(size_t)m * ldq + i];
+    for (int i = tid; i < H * H; i += blockDim.x) s_talk[i] = talk ? talk[i] : ((i / H) == (i % H) ? 1.0f : 0.0f);
+    if (tid < H) {
+        s_max[tid] = sink ? sink[tid] : -INFINITY;
+        s_den[tid] = sink ? 1.0f : 0.0f;
+    }
+    float acc[kWinAcc];
+#pragma unroll
+    for (int r = 0; r < kWinAcc; ++r) acc[r] = 0.0f;
+
+    auto tile_scores = [&](int t0, int nt) {
+        __syncthreads();
+        if (tid < nt) {
+            const int j = j_lo + t0 + tid;
+            s_row[tid] = pages[j / page_tokens] * page_tokens + j % page_tokens;
+        }
+        __syncthreads();
+        for (int idx = tid; idx < H * kWinTile; idx += blockDim.x) {
+            const int h = idx / kWinTile, jj = idx % kWinTile;
+            float s = -INFINITY;
+            if (jj < nt) {
+                const float* kr = cache + (size_t)s_row[jj] * cstride + (size_t)(h / rep) * D;
+                const float* qh = s_q + h * D;
+                float a = 0.0f;
+                for (int d = 0; d < D; ++d) a = fmaf(qh[d], kr[d], a);
+                s = a * scale;
+            }
+            s_s[idx] = s;
+        }
+        __syncthreads();
+    };
+
+    for (int t0 = 0; t0 < n_keys; t0 += kWinTile) {  // pass 1: maximum and denominator per head
+        const int nt = min(kWinTile, n_keys - t0);
+        tile_scores(t0, nt);
+        for (int h = wave; h < H; h += 4) {
+            const float s = s_s[h * kWinTile + lane];
+            const float mo = s_max[h], mn = fmaxf(mo, wave_allmax(s));
+            const float part = wave_allsum(lane < nt ? expf(s - mn) : 0.0f);
+            if (lane == 0) {
+                s_den[h] = s_den[h] * expf(mo - mn) + part;
+                s_max[h] = mn;
+            }
+        }
+    }
+    for (int t0 = 0; t0 < n_keys; t0 += kWinTile) {  // pass 2: weights, their mix, values
+        const int nt = min(kWinTile, n_keys - t0);
+        tile_scores(t0, nt);
+        for (int idx = tid; idx < H * kWinTile; idx += blockDim.x) {
+            const int h = idx / kWinTile, jj = idx % kWinTile;
+            s_s[idx] = jj < nt ? expf(s_s[idx] - s_max[h]) / s_den[h] : 0.0f;
+        }
+        __syncthreads();
+        for (int idx = tid; idx < H * kWinTile; idx += blockDim.x) {
+            const int h = idx / kWinTile, jj = idx % kWinTile;
+            float wsum = 0.0f;
+            for (int g = 0; g < H; ++g) wsum = fmaf(s_talk[h * H + g], s_s[g * kWinTile + jj], wsum);
+            s_w[idx] = wsum;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < kWinAcc; ++r) {
+            const int o = tid + 256 * r;
+            if (o < H * V) {
+                const int h = o / V, c = o % V;
+                const float* vbase = cache + (size_t)G * D + (size_t)(h / rep) * V + c;
+                float a = acc[r];
+                for (int jj = 0; jj < nt; ++jj) a = fmaf(s_w[h * kWinTile + jj], vbase[(size_t)s_row[jj] * cstride], a);
+                acc[r] = a;
+            }
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < kWinAcc; ++r) {
+        const int o = tid + 256 * r;
+        if (o < H * V) s_o[o] = acc[r];
+    }
+    __syncthreads();
+    const float fpos = (float)pos;
+    for (int o = tid; o < H * V; o += blockDim.x) {  // turned back by the query's position
+        const int i = o % V;
+        float sn, cs;
+        sincosf(fpos * vfreq[i >> 1], &sn, &cs);
+        const float own = s_o[o], other = s_o[o - i + (i ^ 1)];
+        out[(size_t)m * ldo + o] = (i & 1) ? own * cs - other * sn : own * cs + other * sn;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------ gated linear recurrent unit
+// Per entry and channel, token by token:  r = sigmoid(gr + br), i = sigmoid(gi + bi), a = exp(-8 r softplus(lam)),
+// S = a S + sqrt(1 - a^2) i u,  out = S * gelu_tanh(y + by).  The loads of a token do not depend on S: eight tokens are
+// requested together.
+__global__ __launch_bounds__(64) void rglru_scan_kernel(const float* u, int ldu, const float* gr, const float* gi, int ldg, const float* br,
+                                                        const float* bi, const float* lam, const float* y, int ldy, const float* by,
+                                                        float* out, int ldo, int C, float* state, size_t slot_stride, const int* ent_start,
+                                                        const int* ent_len, const int* ent_slot) {
+    const int e = blockIdx.x, c = blockIdx.y * blockDim.x + threadIdx.x;
+    if (c >= C) return;
+    const int n = ent_len[e], m0 = ent_start[e];
+    if (n <= 0) return;
+    float* sp = state + (size_t)ent_slot[e] * slot_stride + c;
+    float S = *sp;
+    const float sl = softplus_f(lam[c]), brc = br[c], bic = bi[c], byc = by[c];
+    for (int t0 = 0; t0 < n; t0 += 8) {
+        float uu[8], rr[8], ii[8], yy[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const bool ok = t0 + k < n;
+            const size_t m = (size_t)(m0 + t0 + k);
+            uu[k] = ok ? u[m * ldu + c] : 0.0f;
+            rr[k] = ok ? gr[m * ldg + c] : 0.0f;
+            ii[k] = ok ? gi[m * ldg + c] : 0.0f;
+            yy[k] = ok ? y[m * ldy + c] : 0.0f;
+        }
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            if (t0 + k < n) {
+                const float a = expf(-8.0f * sigmoid_f(rr[k] + brc) * sl);
+                S = fmaf(a, S, sqrtf(1.0f - a * a) * sigmoid_f(ii[k] + bic) * uu[k]);
+                out[(size_t)(m0 + t0 + k) * ldo + c] = S * gelu_tanh_f(yy[k] + byc);
+            }
+        }
+    }
+    *sp = S;
+}
+
+// y = (l / rms(l) * wl + r / rms(r) * wr) / 2, rows of W floats
+__global__ __launch_bounds__(256) void pair_norm_mean_kernel(const float* l, const float* r, const float* wl, const float* wr, float eps, float* y,
+                                                             int W) {
+    __shared__ float s_red[8];
+    const int m = blockIdx.x;
+    const float *lr = l + (size_t)m * W, *rr = r + (size_t)m * W;
+    float sa = 0.0f, sb = 0.0f;
+    for (int i = threadIdx.x; i < W; i += blockDim.x) {
+        sa = fmaf(lr[i], lr[i], sa);
+        sb = fmaf(rr[i], rr[i], sb);
+    }
+    sa = block_allsum(sa, s_red);
+    sb = block_allsum(sb, s_red);
+    const float ra = 1.0f / sqrtf(sa / (float)W + eps), rb = 1.0f / sqrtf(sb / (float)W + eps);
+    for (int i = threadIdx.x; i < W; i += blockDim.x) y[(size_t)m * W + i] = 0.5f * (lr[i] * ra * wl[i] + rr[i] * rb * wr[i]);
+}
+
+// ------------------------------------------------------------------------------------------------ gated delta rule
+// In place on the rows of a step: q and k heads to unit length (q also times dim^-1/2), beta = sigmoid(.), and the decay
+// g = exp(-exp(A_log[h]) * softplus(a + dt_bias)) per head and key channel.  One wave per vector / per stretch of elements.
+__global__ __launch_bounds__(256) void delta_prep_kernel(float* qk, int ldqk, int G, int D, float* beta, int ldb, int H, float* dec, int ldd,
+                                                         const float* a_log, const float* dt_bias) {
+    const int m = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int vsel = wave; vsel < 2 * G; vsel += 4) {  // q heads, then k heads
+        float* p = qk + (size_t)m * ldqk + (size_t)vsel * D;
+        float ss = 0.0f;
+        for (int i = lane; i < D; i += 64) ss = fmaf(p[i], p[i], ss);
+        ss = wave_allsum(ss);
+        const float r = (1.0f / sqrtf(ss + 1e-6f)) * (vsel < G ? 1.0f / sqrtf((float)D) : 1.0f);
+        for (int i = lane; i < D; i += 64) p[i] *= r;
+    }
+    for (int h = threadIdx.x; h < H; h += blockDim.x) beta[(size_t)m * ldb + h] = sigmoid_f(beta[(size_t)m * ldb + h]);
+    for (int i = threadIdx.x; i < H * D; i += blockDim.x) {
+        const float a = expf(a_log[i / D]);
+        dec[(size_t)m * ldd + i] = expf(-a * softplus_f(dec[(size_t)m * ldd + i] + dt_bias[i]));
+    }
+}
+
+// One workgroup per (entry, head); the head's state S[D][V] sits in registers: thread (rg, c) holds rows rg, rg + NR, ... of
+// column c (NR = 256 / VP row groups, VP = the power of two >= V).  Token by token:
+//   S <- g S (rows);  kv = S^T k;  u = beta (v - kv);  S <- S + k u^T;  o = S^T q
+// The two column sums meet in the LDS; the token's vectors are fetched one token ahead.
+template <int RPT>
+__global__ __launch_bounds__(256) void delta_scan_kernel(const float* qk, int ldqk, const float* v, int ldv, const float* beta, int ldb,
+                                                         const float* dec, int ldd, float* out, int ldo, int H, int G, int D, int V, int VP,
+                                                         float* state, size_t slot_stride, const int* ent_start, const int* ent_len,
+                                                         const int* ent_slot) {
+    extern __shared__ __attribute__((aligned(16))) float s_delta[];
+    const int NR = 256 / VP;
+    const int n_stage = 3 * D + V + 1;      // q | k | g | v | beta
+    float* s_stage = s_delta;               // [2][n_stage]
+    float* s_p1 = s_stage + 2 * n_stage;    // [NR][VP]
+    float* s_p2 = s_p1 + NR * VP;           // [NR][VP]
+    const int e = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+    const int n = ent_len[e], m0 = ent_start[e];
+    if (n <= 0) return;
+    const int c = tid % VP, rg = tid / VP, kvh = h / (H / G);
+    const bool col_ok = c < V;
+    float* Sg = state + (size_t)ent_slot[e] * slot_stride + (size_t)h * D * V;
+    float S[RPT];
+#pragma unroll
+    for (int r = 0; r < RPT; ++r) {
+        const int d = rg + NR * r;
+        S[r] = (col_ok && d < D) ? Sg[(size_t)d * V + c] : 0.0f;
+    }
+    constexpr int kPre = 5;  // 256 * 5 >= 3 * 256 + 256 + 1
+    auto fetch = [&](int t, float pre[kPre]) {
+        const size_t m = (size_t)(m0 + t);
+#pragma unroll
+        for (int i = 0; i < kPre; ++i) {
+            const int idx = tid + 256 * i;
+            float val = 0.0f;
+            if (idx < D) val = qk[m * ldqk + (size_t)kvh * D + idx];
+            else if (idx < 2 * D) val = qk[m * ldqk + (size_t)(G + kvh) * D + (idx - D)];
+            else if (idx < 3 * D) val = dec[m * ldd + (size_t)h * D + (idx - 2 * D)];
+            else if (idx < 3 * D + V) val = v[m * ldv + (size_t)h * V + (idx - 3 * D)];
+            else if (idx == 3 * D + V) val = beta[m * ldb + h];
+            pre[i] = val;
+        }
+    };
+    auto stash = [&](int buf, const float pre[kPre]) {
+#pragma unroll
+        for (int i = 0; i < kPre; ++i) {
+            const int idx = tid + 256 * i;
+            if (idx < n_stage) s_stage[buf * n_stage + idx] = pre[i];
+        }
+    };
+    float pre[kPre];
+    fetch(0, pre);
+    stash(0, pre);
+    for (int t = 0; t < n; ++t) {
+        if (t + 1 < n) fetch(t + 1, pre);
+        __syncthreads();  // the token's vectors are staged
+        const float* sq = s_stage + (t & 1) * n_stage;
+        const float *sk = sq + D, *sg = sk + D, *sv = sg + D;
+        const float bt = sv[V];
+        float part = 0.0f;
+#pragma unroll
+        for (int r = 0; r < RPT; ++r) {
+            const int d = rg + NR * r;
+            if (d < D) {
+                S[r] *= sg[d];
+                part = fmaf(S[r], sk[d], part);
+            }
+        }
+        s_p1[rg * VP + c] = part;
+        __syncthreads();
+        float kv = 0.0f;
+        for (int g2 = 0; g2 < NR; ++g2) kv += s_p1[g2 * VP + c];
+        const float u = col_ok ? bt * (sv[c] - kv) : 0.0f;
+        float part2 = 0.0f;
+#pragma unroll
+        for (int r = 0; r < RPT; ++r) {
+            const int d = rg + NR * r;
+            if (d < D) {
+                S[r] = fmaf(sk[d], u, S[r]);
+                part2 = fmaf(S[r], sq[d], part2);
+            }
+        }
+        s_p2[rg * VP + c] = part2;
+        if (t + 1 < n) stash((t + 1) & 1, pre);
+        __syncthreads();
+        if (rg == 0 && col_ok) {
+            float o = 0.0f;
+            for (int g2 = 0; g2 < NR; ++g2) o += s_p2[g2 * VP + c];
+            out[(size_t)(m0 + t) * ldo + (size_t)h * V + c] = o;
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < RPT; ++r) {
+        const int d = rg + NR * r;
+        if (col_ok && d < D) Sg[(size_t)d * V + c] = S[r];
+    }
+}
+
+// one wave per (row, head) vector, in place: v / rms(v) * w * sigmoid(gate)
+__global__ __launch_bounds__(256) void norm_gate_kernel(float* v, int ld, int rows_per_m, int width, int n_vec, const float* w, float eps,
+                                                        const float* gate, int ldg) {
+    const int vec = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    if (vec >= n_vec) return;
+    const size_t m = vec / rows_per_m, hh = vec % rows_per_m;
+    float* p = v + m * ld + hh * width;
+    const float* gp = gate + m * ldg + hh * width;
+    float ss = 0.0f;
+    for (int i = lane; i < width; i += 64) ss = fmaf(p[i], p[i], ss);
+    ss = wave_allsum(ss);
+    const float r = 1.0f / sqrtf(ss / (float)width + eps);
+    for (int i = lane; i < width; i += 64) p[i] = p[i] * r * w[i] * sigmoid_f(gp[i]);
+}
+
+}  // namespace
+
+int launch_add_rows(float* x, const float* y, int M, int W, hipStream_t s) {
+    const size_t n = (size_t)M * W;
+    if (n == 0) return ZG_OK;
+    add_rows_kernel<<<(unsigned)((n + 255) / 256), 256, 0, s>>>(x, y, n);
+    ZG_HIP(hipGetLastError());
+    return ZG_OK;
+}
+
+int launch_causal_conv(const ConvArgs& a, int M, int n_entries, const int* row_off, const int* row_slot, const int* ent_start, const int* ent_len,
+                       const int* ent_slot, hipStream_t s) {
+    if (M <= 0 || a.C <= 0) return ZG_OK;
+    ZG_REQUIRE(a.taps >= 1 && a.taps <= kMaxTaps, ZG_ERR_UNSUPPORTED, "convolution: %d taps (1 to %d)", a.taps, kMaxTaps);
+    ZG_REQUIRE(a.in != a.out, ZG_ERR_ARG, "convolution: in place");
+    const int bx = a.C >= 256 ? 256 : 64;
+    causal_conv_kernel<<<dim3(M, (a.C + bx - 1) / bx), bx, 0, s>>>(a.in, a.ld_in, a.out, a.ld_out, a.C, a.taps, a.w, a.bias, a.pre_bias, a.flags, a.tail,
+                                                                 a.slot_stride, row_off, row_slot);
+    ZG_HIP(hipGetLastError());
+    if (a.taps > 1) {
+        conv_tail_kernel<<<dim3(n_entries, (a.C + bx - 1) / bx), bx, 0, s>>>(a.in, a.ld_in, a.C, a.taps, a.pre_bias, a.tail, a.slot_stride, ent_start,
+                                                                           ent_len, ent_slot);
+        ZG_HIP(hipGetLastError());
+    }
+    return ZG_OK;
+}
+
+int launch_window_prep(float* proj, int ld, int M, int H, int G, int D, int V, Rotary rot, const float* vfreq, const int* row_pos,
+                       const int* row_slot, const int* page_table, int max_pages, int page_tokens, float* cache, hipStream_t s) {
+    if (M <= 0) return ZG_OK;
+    ZG_REQUIRE(V % 2 == 0 && rot.dims % 2 == 0 && rot.dims <= D, ZG_ERR_ARG, "windowed attention: %d value channels, %d of %d rotated", V, rot.dims, D);
+    window_prep_kernel<<<M, 256, 0, s>>>(proj, ld, H, G, D, V, rot, vfreq, row_pos, row_slot, page_table, max_pages, page_tokens, cache);
+    ZG_HIP(hipGetLastError());
+    return ZG_OK;
+}
+
+int launch_window_attention(const float* q, int ldq, float* out, int ldo, int M, int H, int G, int D, int V, float scale, int window,
+                            const float* sink, const float* talk, const float* vfreq, const int* row_pos, const int* row_slot,
+                            const int* page_table, int max_pages, int page_tokens, const float* cache, hipStream_t s) {
+    if (M <= 0) return ZG_OK;
+    ZG_REQUIRE(H >= 1 && H <= kWinMaxHeads && G >= 1 && H % G == 0, ZG_ERR_UNSUPPORTED, "windowed attention: %d heads on %d key heads (at most %d heads)",
+               H, G, kWinMaxHeads);
+    ZG_REQUIRE(H * V <= 256 * kWinAcc, ZG_ERR_UNSUPPORTED, "windowed attention: %d heads x %d value channels (at most %d together)", H, V,
+               256 * kWinAcc);
+    const size_t lds = ((size_t)H * D + 2 * (size_t)H * kWinTile + (size_t)H * H + (size_t)H * V) * sizeof(float);
+    ZG_REQUIRE(lds <= 60 * 1024, ZG_ERR_UNSUPPORTED, "windowed attention: %d heads of %d + %d channels need %zu bytes of LDS", H, D, V, lds);
+    window_attention_kernel<<<M, 256, lds, s>>>(q, ldq, out, ldo, H, G, D, V, scale, window, sink, talk, vfreq, row_pos, row_slot, page_table,
+                                                max_pages, page_tokens, cache);
+    ZG_HIP(hipGetLastError());
+    return ZG_OK;
+}
+
+int launch_rglru_scan(const float* u, int ldu, const float* gr, const float* gi, int ldg, const float* br, const float* bi, const float* lam,
+                      const float* y, int ldy, const float* by, float* out, int ldo, int C, float* state, size_t slot_stride, const int* ent_start,
+                      const int* ent_len, const int* ent_slot, int n_entries, hipStream_t s) {
+    if (n_entries <= 0 || C <= 0) return ZG_OK;
+    rglru_scan_kernel<<<dim3(n_entries, (C + 63) / 64), 64, 0, s>>>(u, ldu, gr, gi, ldg, br, bi, lam, y, ldy, by, out, ldo, C, state, slot_stride,
+                                                                  ent_start, ent_len, ent_slot);
+    ZG_HIP(hipGetLastError());
+    return ZG_OK;
+}
+
+int launch_pair_norm_mean(const float* l, const float* r, const float* wl, const float* wr, float eps, float* y, int M, int W, hipStream_t s) {
+    if (M <= 0) return ZG_OK;
+    pair_norm_mean_kernel<<<M, 256, 0, s>>>(l, r, wl, wr, eps, y, W);
+    ZG_HIP(hipGetLastError());
+    return ZG_OK;
+}
+
+int launch_delta_prep(float* qk, int ldqk, int G, int D, float* beta, int ldb, int H, float* dec, int ldd, const float* a_log,
+                      const float* dt_bias, int M, hipStream_t s) {
+    if (M <= 0) return ZG_OK;
+    delta_prep_kernel<<<M, 256, 0, s>>>(qk, ldqk, G, D, beta, ldb, H, dec, ldd, a_log, dt_bias);
+    ZG_HIP(hipGetLastError());
+    return ZG_OK;
+}
+
+int launch_delta_scan(const float* qk, int ldqk, const float* v, int ldv, const float* beta, int ldb, const float* dec, int ldd, float* out,
+                      int ldo, int H, int G, int D, int V, float* state, size_t slot_stride, const int* ent_start, const int* ent_len,
+                      const int* ent_slot, int n_entries, hipStream_t s) {
+    if (n_entries <= 0) return ZG_OK;
+    ZG_REQUIRE(D >= 1 && D <= 256 && V >= 1 && V <= 256 && G >= 1 && H % G == 0, ZG_ERR_UNSUPPORTED,
+               "delta rule: %d heads on %d key heads, %d key and %d value channels per head (at most 256 each)", H, G, D, V);
+    int VP = 1;
+    while (VP < V) VP <<= 1;
+    const int NR = 256 / VP, rpt = (D + NR - 1) / NR;
+    ZG_REQUIRE(rpt <= 64, ZG_ERR_UNSUPPORTED, "delta rule: a state of %d x %d per head (at most 16384 elements)", D, V);
+    const size_t lds = (2 * (size_t)(3 * D + V + 1) + 2 * 256) * sizeof(float);
+    const dim3 grid(n_entries, H);
+#define ZG_DELTA(R)                                                                                                                          \
+    delta_scan_kernel<R><<<grid, 256, lds, s>>>(qk, ldqk, v, ldv, beta, ldb, dec, ldd, out, ldo, H, G, D, V, VP, state, slot_stride, ent_start, \
+                                                ent_len, ent_slot)
+    if (rpt <= 4) ZG_DELTA(4);
+    else if (rpt <= 8) ZG_DELTA(8);
+    else if (rpt <= 16) ZG_DELTA(16);
+    else if (rpt <= 32) ZG_DELTA(32);
+    else ZG_DELTA(64);
+#undef ZG_DELTA
+    ZG_HIP(hipGetLastError());
+    return ZG_OK;
+}
+
+int launch_norm_gate(float* v, int ld, int rows_per_m, int width, int M, const float* w, float eps, const float* gate, int ldg, hipStream_t s) {
+    const int n_vec = M * rows_per_m;
+    if (n_vec <= 0) return ZG_OK;
+    norm_gate_kernel<<<(n_vec + 3) / 4, 256, 0, s>>>(v, ld, rows_per_m, width, n_vec, w, eps, gate, ldg);
+    ZG_HIP(hipGetLastError());
+    return ZG_OK;
+}
+
+}  // namespace lm
+}  // namespace zg

@@ -6,9 +6,15 @@ library runs whatever list it is given.  This module turns a checkpoint's config
 any number of tokens at a time (several sequences per step), and closed; `generate` runs prompts through the same step with
 the library's greedy / sampling head.
 
-config.json of the Tokosun design (the only architecture of the family so far; zig_gpt2_amd/models.py maps names to classes):
-  vocab, width, norm.eps, layers[i] = {type: "hgrn2" | "latent_attention", mixer: {...sizes...}, mlp: null | {kind: "dense", ff}
+config.json (zig_gpt2_amd/models.py maps architecture names to loaders; `DESIGNS` below holds what a name fixes):
+  vocab, width, norm.eps, layers[i] = {type, mixer: {...sizes...}, mlp: null | {kind: "dense", ff}
   | {kind: "moe", expert: {ff}, router: {experts, top}}}, loop: null | {start, stop, times}.
+  Tokosun: type "hgrn2" | "latent_attention"; token shift in front of the mixer; gated experts, softmax router with correction.
+  Gupizen: type "parallel" (mixer.left: windowed attention with sink, mixed heads and rotated values; mixer.right: gated linear
+  recurrent unit) | "channel_delta" (gated delta rule); canon.taps: input convolution of both sublayers; embedding.scale; tied
+  head; the embedding output added again in front of every repetition of the loop but the first; plain gelu experts, the
+  router's largest logits.  Sizes the configuration does not list (the inner sizes of two-step projections) come from the
+  checkpoint's tensor shapes.
 """
 import ctypes as C
 import json
@@ -21,7 +27,17 @@ import numpy as np
 from . import _lib
 from ._lib import check_lm as check
 
-MIXERS = {"hgrn2": _lib.LM_MIX_HGRN2, "latent_attention": _lib.LM_MIX_LATENT_ATTENTION}
+MIXERS = {"hgrn2": _lib.LM_MIX_HGRN2, "latent_attention": _lib.LM_MIX_LATENT_ATTENTION, "parallel": _lib.LM_MIX_PARALLEL,
+          "channel_delta": _lib.LM_MIX_CHANNEL_DELTA}
+ROT_STYLES = {"yarn": _lib.LM_ROT_YARN, "bands": _lib.LM_ROT_BANDS}
+EXPERT_ACTS = {"glu_silu": _lib.LM_ACT_GLU_SILU, "gelu": _lib.LM_ACT_GELU}
+ROUTERS = {"softmax_all": _lib.LM_ROUTE_SOFTMAX_ALL, "top_logits": _lib.LM_ROUTE_TOP_LOGITS}
+
+# what an architecture name fixes beyond config.json
+DESIGNS = {
+    "Tokosun": dict(mixers=("hgrn2", "latent_attention"), tied_head=False, loop_readd=False, expert_act="glu_silu", router="softmax_all"),
+    "Gupizen": dict(mixers=("parallel", "channel_delta"), tied_head=True, loop_readd=True, expert_act="gelu", router="top_logits"),
+}
 
 
 @dataclass
@@ -39,17 +55,50 @@ class LayerSpec:
     rot_dims: int = 0
     rot_base: float = 10000.0
     rot_scaling: Optional[dict] = None  # {factor, original, fast, slow}
+    rot_style: str = "yarn"  # yarn: {factor, original, fast, slow} | bands: {factor, original, low, high}
     ff: str = "none"  # none | dense | moe
     ff_width: int = 0
     experts: int = 0
     top: int = 0
+    expert_act: str = "glu_silu"
+    router: str = "softmax_all"
+    kv_heads: int = 0
+    window: int = 0
+    lru_width: int = 0
+    lru_blocks: int = 0
+    lru_conv: int = 0
+    conv: int = 0
+    decay_rank: int = 0
+    gate_rank: int = 0
 
     @classmethod
-    def from_json(cls, entry):
+    def from_json(cls, entry, design="Tokosun", shapes=None, prefix=""):
+        """entry: one element of config['layers'].  shapes: {tensor name: shape} of the checkpoint, for the sizes that only
+        tensor shapes give (prefix: 'l<i>.')."""
         kind, m = entry["type"], entry["mixer"]
-        if kind not in MIXERS:
-            raise ValueError(f"unknown mixer type {kind!r} (known: {sorted(MIXERS)})")
-        kw = dict(mixer=kind, heads=int(m["heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]))
+        fixed = DESIGNS[design]
+        if kind not in fixed["mixers"]:
+            raise ValueError(f"unknown mixer type {kind!r} (known to {design}: {sorted(fixed['mixers'])})")
+        if kind == "parallel":
+            l, r = m["left"], m["right"]
+            rot = l.get("rot") or {}
+            kw = dict(mixer=kind, heads=int(l["heads"]), kv_heads=int(l.get("kv_heads", l["heads"])), dim=int(l["dim"]), vdim=int(l["vdim"]),
+                      scale=float(l["scale"]), window=int((l.get("mask") or {}).get("size", 0)), rot_dims=int(rot.get("dims", 0)),
+                      rot_base=float(rot.get("base", 10000.0)), rot_scaling=dict(rot["scaling"]) if rot.get("scaling") else None,
+                      rot_style="bands", lru_width=int(r["width"]), lru_blocks=int(r["blocks"]), lru_conv=int(r["conv"]))
+        elif kind == "channel_delta":
+            def inner(key, tensor):
+                if key in m:
+                    return int(m[key])
+                if shapes is None or prefix + tensor not in shapes:
+                    raise KeyError(f"{prefix}mix: the inner size {key!r} needs the shape of tensor {prefix + tensor!r}")
+                return int(shapes[prefix + tensor][0])
+
+            kw = dict(mixer=kind, heads=int(m["heads"]), kv_heads=int(m.get("kv_heads", m["heads"])), dim=int(m["dim"]), vdim=int(m["vdim"]),
+                      conv=int(m["conv"]), decay_rank=inner("decay_rank", "mix.a1"), gate_rank=inner("gate_rank", "mix.g1"))
+        else:
+            kw = dict(mixer=kind, heads=int(m["heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]))
+        kw.update(expert_act=fixed["expert_act"], router=fixed["router"])
         if kind == "latent_attention":
             rot = m.get("rot") or {}
             kw.update(rot_dim=int(m["rot_dim"]), kv_rank=int(m["kv_rank"]), q_rank=int(m["q_rank"]), scale=float(m["scale"]),
@@ -67,6 +116,16 @@ class LayerSpec:
 
     def to_json(self):
         mixer = {"heads": self.heads, "dim": self.dim, "vdim": self.vdim}
+        if self.mixer == "parallel":
+            rot = {"base": self.rot_base, "dims": self.rot_dims}
+            if self.rot_scaling:
+                rot["scaling"] = dict(self.rot_scaling)
+            left = dict(mixer, kv_heads=self.kv_heads, scale=self.scale, rot=rot)
+            if self.window:
+                left["mask"] = {"size": self.window}
+            mixer = {"left": left, "right": {"width": self.lru_width, "blocks": self.lru_blocks, "conv": self.lru_conv}}
+        elif self.mixer == "channel_delta":
+            mixer.update(kv_heads=self.kv_heads, conv=self.conv, decay_rank=self.decay_rank, gate_rank=self.gate_rank)
         if self.mixer == "latent_attention":
             rot = {"base": self.rot_base, "dims": self.rot_dims}
             if self.rot_scaling:
@@ -81,21 +140,43 @@ class LayerSpec:
 
     def to_c(self):
         sc = self.rot_scaling or {}
+        bands = self.rot_style == "bands"  # the bands' `high` / `low` travel in the fields of the blend's `fast` / `slow`
         return _lib.LmLayer(MIXERS[self.mixer], self.heads, self.dim, self.vdim, self.rot_dim, self.kv_rank, self.q_rank, self.scale, self.rot_dims,
-                            self.rot_base, 1 if self.rot_scaling else 0, float(sc.get("factor", 1.0)), float(sc.get("original", 1.0)),
-                            float(sc.get("fast", 1.0)), float(sc.get("slow", 1.0)),
+                            self.rot_base, ROT_STYLES[self.rot_style] if self.rot_scaling else 0, float(sc.get("factor", 1.0)),
+                            float(sc.get("original", 1.0)), float(sc.get("high" if bands else "fast", 1.0)),
+                            float(sc.get("low" if bands else "slow", 1.0)),
                             {"none": _lib.LM_FF_NONE, "dense": _lib.LM_FF_DENSE, "moe": _lib.LM_FF_MOE}[self.ff], self.ff_width, self.experts,
-                            self.top)
+                            self.top, self.kv_heads, self.window, self.lru_width, self.lru_blocks, self.lru_conv, self.conv, self.decay_rank,
+                            self.gate_rank, EXPERT_ACTS[self.expert_act], ROUTERS[self.router])
 
-    def tensor_shapes(self, prefix, width):
+    def tensor_shapes(self, prefix, width, canon_taps=0):
         """{checkpoint tensor name: shape} of this layer."""
         H, D, V, W = self.heads, self.dim, self.vdim, width
-        t = {prefix + "norm1": (W,), prefix + "norm1b": (W,), prefix + "shift": (W,)}
+        t = {prefix + "norm1": (W,), prefix + "norm1b": (W,)}
+        if canon_taps:
+            t[prefix + "canon1"] = (W, canon_taps)
+            if self.ff != "none":
+                t[prefix + "canon2"] = (W, canon_taps)
+        else:
+            t[prefix + "shift"] = (W,)
         m = prefix + "mix."
-        if self.mixer == "hgrn2":
+        if self.mixer == "parallel":
+            G, C, NB = self.kv_heads, self.lru_width, self.lru_blocks
+            l, r = m + "left.", m + "right."
+            t.update({l + "q": (H * D, W), l + "k": (G * D, W), l + "v": (G * V, W), l + "talk": (H, H), l + "sink": (H,), l + "o": (W, H * V),
+                      l + "out": (W,), r + "out": (W,), r + "y": (C, W), r + "y.b": (C,), r + "x": (C, W), r + "x.b": (C,),
+                      r + "conv": (C, self.lru_conv), r + "conv.b": (C,), r + "ra": (NB, C // NB, C // NB), r + "ra.b": (NB, C // NB),
+                      r + "ri": (NB, C // NB, C // NB), r + "ri.b": (NB, C // NB), r + "lam": (C,), r + "o": (W, C)})
+        elif self.mixer == "channel_delta":
+            G = self.kv_heads
+            t.update({m + "q": (G * D, W), m + "q.conv": (G * D, self.conv), m + "k": (G * D, W), m + "k.conv": (G * D, self.conv),
+                      m + "v": (H * V, W), m + "v.conv": (H * V, self.conv), m + "b": (H, W), m + "A_log": (H,), m + "norm": (V,),
+                      m + "a1": (self.decay_rank, W), m + "a2": (H * D, self.decay_rank), m + "dt_bias": (H * D,),
+                      m + "g1": (self.gate_rank, W), m + "g2": (H * V, self.gate_rank), m + "o": (W, H * V)})
+        elif self.mixer == "hgrn2":
             t.update({m + "q": (H * D, W), m + "f": (H * D, W), m + "f.b": (H * D,), m + "lower": (H * D,), m + "v": (H * V, W), m + "norm": (V,),
                       m + "o": (W, H * V)})
-        else:
+        elif self.mixer == "latent_attention":
             R, KR, QR = self.rot_dim, self.kv_rank, self.q_rank
             t.update({m + "dq": (QR, W), m + "dq.norm": (QR,), m + "uq": (H * (D + R), QR), m + "dkv": (KR + R, W), m + "dkv.norm": (KR,),
                       m + "uk": (H * D, KR), m + "uv": (H * V, KR), m + "o": (W, H * V)})
@@ -106,8 +187,10 @@ class LayerSpec:
             t.update({f + "up": (self.ff_width, W), f + "down": (W, self.ff_width)})
         elif self.ff == "moe":
             for e in range(self.experts):
-                t.update({f"{f}e{e}.gate": (self.ff_width, W), f"{f}e{e}.up": (self.ff_width, W), f"{f}e{e}.down": (W, self.ff_width)})
-            t.update({f + "router": (self.experts, W), f + "correction": (self.experts,)})
+                t.update({f"{f}e{e}.up": (self.ff_width, W), f"{f}e{e}.down": (W, self.ff_width)})
+                if self.expert_act == "glu_silu":
+                    t[f"{f}e{e}.gate"] = (self.ff_width, W)
+            t.update({f + "router": (self.experts, W), f + ("router.b" if self.router == "top_logits" else "correction"): (self.experts,)})
         return t
 
 
@@ -119,22 +202,47 @@ class LMConfig:
     norm_eps: float = 1e-6
     loop: Optional[dict] = None  # {start, stop, times}
     architecture: str = "Tokosun"
+    embed_scale: float = 1.0
+    canon_taps: int = 0  # > 0: both sublayers read h + conv(h) over this many tokens; 0: token shift in front of the mixer
     extra: dict = field(default_factory=dict)
 
     @classmethod
-    def from_json(cls, cfg):
-        return cls(vocab=int(cfg["vocab"]), width=int(cfg["width"]), layers=[LayerSpec.from_json(e) for e in cfg["layers"]],
-                   norm_eps=float(cfg["norm"]["eps"]), loop=dict(cfg["loop"]) if cfg.get("loop") else None,
-                   architecture=cfg.get("architecture", "Tokosun"))
+    def from_json(cls, cfg, shapes=None):
+        """cfg: the dict of config.json; shapes: {tensor name: shape} of the checkpoint (for sizes only shapes give)."""
+        arch = cfg.get("architecture", "Tokosun")
+        if arch not in DESIGNS:
+            raise ValueError(f"architecture {arch!r} is not a layered design (known: {sorted(DESIGNS)})")
+        layers = [LayerSpec.from_json(e, arch, shapes, f"l{i}.") for i, e in enumerate(cfg["layers"])]
+        return cls(vocab=int(cfg["vocab"]), width=int(cfg["width"]), layers=layers,
+                   norm_eps=float(cfg["norm"]["eps"]), loop=dict(cfg["loop"]) if cfg.get("loop") else None, architecture=arch,
+                   embed_scale=float((cfg.get("embedding") or {}).get("scale", 1.0)), canon_taps=int((cfg.get("canon") or {}).get("taps", 0)))
 
     @classmethod
     def from_dir(cls, path):
+        from . import weights_io
+
         with open(os.path.join(path, "config.json")) as f:
-            return cls.from_json(json.load(f))
+            cfg = json.load(f)
+        st = os.path.join(path, "model.safetensors")
+        shapes = {k: tuple(a.shape) for k, (_, a) in weights_io.read_safetensors(st).items()} if os.path.exists(st) else None
+        return cls.from_json(cfg, shapes)
 
     def to_json(self):
-        return {"architecture": self.architecture, "vocab": self.vocab, "width": self.width, "norm": {"eps": self.norm_eps},
-                "layers": [l.to_json() for l in self.layers], "loop": dict(self.loop) if self.loop else None}
+        out = {"architecture": self.architecture, "vocab": self.vocab, "width": self.width, "norm": {"eps": self.norm_eps},
+               "layers": [l.to_json() for l in self.layers], "loop": dict(self.loop) if self.loop else None}
+        if self.embed_scale != 1.0:
+            out["embedding"] = {"scale": self.embed_scale}
+        if self.canon_taps:
+            out["canon"] = {"taps": self.canon_taps}
+        return out
+
+    @property
+    def tied_head(self):
+        return DESIGNS[self.architecture]["tied_head"]
+
+    def flags(self):
+        d = DESIGNS[self.architecture]
+        return (_lib.LM_TIED_HEAD if d["tied_head"] else 0) | (_lib.LM_LOOP_READD if d["loop_readd"] else 0)
 
     def passes(self):
         """Layer index of every pass, in execution order."""
@@ -145,9 +253,11 @@ class LMConfig:
         return list(range(a)) + list(range(a, b)) * k + list(range(b, n))
 
     def tensor_shapes(self):
-        t = {"embed": (self.vocab, self.width), "head": (self.vocab, self.width), "final.norm": (self.width,)}
+        t = {"embed": (self.vocab, self.width), "final.norm": (self.width,)}
+        if not self.tied_head:
+            t["head"] = (self.vocab, self.width)
         for i, l in enumerate(self.layers):
-            t.update(l.tensor_shapes(f"l{i}.", self.width))
+            t.update(l.tensor_shapes(f"l{i}.", self.width, self.canon_taps))
         return t
 
 
@@ -164,7 +274,8 @@ class LayeredLM:
         loop = config.loop or {"start": 0, "stop": 0, "times": 1}
         cfg = _lib.LmConfig(config.vocab, config.width, len(config.layers), self._layers, int(loop["start"]), int(loop["stop"]), int(loop["times"]),
                             config.norm_eps, max_tokens, max_seqs, max_step_tokens, page_tokens,
-                            (_lib.LM_F32 if dtype == "float32" else 0) | (0 if use_graph else _lib.LM_NO_GRAPH))
+                            (_lib.LM_F32 if dtype == "float32" else 0) | (0 if use_graph else _lib.LM_NO_GRAPH) | config.flags(),
+                            config.embed_scale, config.canon_taps)
         h = C.c_void_p()
         check(L.zg_lm_create(C.byref(h), C.byref(cfg), device))
         self.h = h
@@ -356,9 +467,10 @@ class Scheduler:
                 else:
                     entries.append((r["seq"], [r["out"][-1]], [0]))
                     asked.append(r)
-            before = self.model.free_tokens()
+            before = {r["seq"]: self.model.seq_len(r["seq"]) for r in self.active}
             logits = self.model.step(entries)
-            self._reserved -= before - self.model.free_tokens()  # pages the step took are no longer merely promised
+            for r in self.active:  # pages the step took are no longer merely promised (a windowed model may have given others back)
+                self._reserved -= (-(-self.model.seq_len(r["seq"]) // self.page) - -(-before[r["seq"]] // self.page)) * self.page
             self.steps += 1
             for r, row in zip(asked, logits):
                 r["out"].append(self._choose(r, row))
