@@ -87,6 +87,8 @@ struct Slot {
     bool open = false;
     size_t len = 0;
     std::vector<int> pages;  // by position / page_tokens; -1: returned to the pool (behind every window)
+    std::vector<int> ring;   // the device's view: page of position p at ring[(p / page_tokens) % max_pages]
+    size_t first_live = 0;   // pages in front of this one have been returned
 };
 
 struct Bump {
@@ -774,7 +776,7 @@ int run_portion(zg_lm* g, const std::vector<Piece>& pieces, float* logits_out, c
         }
         for (auto& w : pc.wants) wants.push_back({ent_start[e] + w.first, w.second});
         const Slot& sl = g->slots[pc.slot];
-        ZG_HIP(hipMemcpyAsync(g->page_table + (size_t)pc.slot * g->max_pages, sl.pages.data(), sl.pages.size() * sizeof(int), hipMemcpyHostToDevice, s));
+        ZG_HIP(hipMemcpyAsync(g->page_table + (size_t)pc.slot * g->max_pages, sl.ring.data(), sl.ring.size() * sizeof(int), hipMemcpyHostToDevice, s));
     }
     ZG_HIP(hipMemcpyAsync(g->meta, g->h_meta, meta_ints(g) * sizeof(int), hipMemcpyHostToDevice, s));
     const int* d_want = g->meta + 5 * (size_t)MS;
@@ -872,8 +874,8 @@ int step_impl(zg_lm* g, const zg_lm_entry* entries, size_t n_entries, float* log
         n_want += e.n_want;
         const Slot& sl = g->slots[e.seq];
         const size_t pages = (sl.len + e.n_tokens + g->P - 1) / g->P;
-        ZG_REQUIRE(pages <= (size_t)g->max_pages, ZG_ERR_SHAPE, "lm_step: sequence %d would hold %zu tokens (at most %zu)", e.seq, sl.len + e.n_tokens,
-                   (size_t)g->max_pages * g->P);
+        ZG_REQUIRE(pages - sl.first_live <= (size_t)g->max_pages, ZG_ERR_SHAPE, "lm_step: sequence %d would hold %zu tokens in the cache (at most %zu)",
+                   e.seq, sl.len + e.n_tokens - sl.first_live * g->P, (size_t)g->max_pages * g->P);
         need_pages += pages > sl.pages.size() ? pages - sl.pages.size() : 0;
     }
     ZG_REQUIRE(need_pages <= g->free_pages.size(), ZG_ERR_SHAPE, "lm_step: %zu cache pages needed, %zu free (max_tokens %zu)", need_pages,
@@ -884,6 +886,7 @@ int step_impl(zg_lm* g, const zg_lm_entry* entries, size_t n_entries, float* log
         Slot& sl = g->slots[entries[i].seq];
         const size_t pages = (sl.len + entries[i].n_tokens + g->P - 1) / g->P;
         while (sl.pages.size() < pages) {
+            sl.ring[sl.pages.size() % g->max_pages] = g->free_pages.back();
             sl.pages.push_back(g->free_pages.back());
             g->free_pages.pop_back();
         }
@@ -929,6 +932,7 @@ int step_impl(zg_lm* g, const zg_lm_entry* entries, size_t n_entries, float* log
                     g->free_pages.push_back(sl.pages[pg]);
                     sl.pages[pg] = -1;
                 }
+            sl.first_live = std::max(sl.first_live, std::min(dead, sl.pages.size()));
         }
     return ZG_OK;
 }
@@ -1179,6 +1183,8 @@ int zg_lm_seq_open(zg_lm* g, int* seq_out) {
     sl.open = true;
     sl.len = 0;
     sl.pages.clear();
+    sl.ring.assign(g->max_pages, 0);
+    sl.first_live = 0;
     *seq_out = sidx;
     return ZG_OK;
 }

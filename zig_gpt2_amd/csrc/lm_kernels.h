@@ -138,7 +138,8 @@ int launch_add_rows(float* x, const float* y, int M, int W, hipStream_t s);
 
 // ------------------------------------------------------------------------------------------------ windowed attention (sink, mixed heads, rotated values)
 // proj rows [q (H D) | k (G D) | v (G V)]: q rotated in place; the rotated key and the value rotated over all V channels (pair i by
-// pos * vfreq[i]) written to the token's cache row [G D | G V] (cache row of (slot, pos) through the page table).
+// pos * vfreq[i]) written to the token's cache row [G D | G V]; the page of (slot, pos) is page_table[slot][(pos / P) % max_pages]:
+// a ring, so that a sequence whose old pages have been given back can grow beyond max_pages * P positions.
 int launch_window_prep(float* proj, int ld, int M, int H, int G, int D, int V, Rotary rot, const float* vfreq, const int* row_pos,
                        const int* row_slot, const int* page_table, int max_pages, int page_tokens, float* cache, hipStream_t s);
 // out[m][h] = turn_back_pos( sum_j w_h(j) value_(h / (H/G))(j) ),  w_h = sum_g talk[h][g] p_g,

@@ -94,7 +94,7 @@ __global__ __launch_bounds__(256) void window_prep_kernel(float* proj, int ld, i
                                                           int page_tokens, float* cache) {
     const int m = blockIdx.x;
     const int pos = row_pos[m];
-    const int page = page_table[(size_t)row_slot[m] * max_pages + pos / page_tokens];
+    const int page = page_table[(size_t)row_slot[m] * max_pages + (pos / page_tokens) % max_pages];
     float* crow = cache + ((size_t)page * page_tokens + pos % page_tokens) * ((size_t)G * (D + V));
     float* row = proj + (size_t)m * ld;
     const float fpos = (float)pos;
@@ -174,7 +174,7 @@ __global__ __launch_bounds__(256) void window_attention_kernel(const float* q, i
         __syncthreads();
         if (tid < nt) {
             const int j = j_lo + t0 + tid;
-            s_row[tid] = pages[j / page_tokens] * page_tokens + j % page_tokens;
+            s_row[tid] = pages[(j / page_tokens) % max_pages] * page_tokens + j % page_tokens;
         }
         __syncthreads();
         for (int idx = tid; idx < H * kWinTile; idx += blockDim.x) {

@@ -140,11 +140,38 @@ inline std::string slurp(const std::string& path, size_t max_bytes = (size_t)-1)
     return s;
 }
 
-// config.json of the Tokosun design -> layer descriptors (the keys zig_gpt2_amd/lm.py reads)
-inline void build_config(const Json& cfg, std::vector<zg_lm_layer>& layers, zg_lm_config& out) {
+// the JSON header of a safetensors file (name -> dtype, shape, data_offsets)
+inline Json safetensors_header(const std::string& path) {
+    std::ifstream f(path, std::ios::binary);
+    if (!f) throw std::runtime_error("cannot open " + path);
+    uint64_t n = 0;
+    f.read(reinterpret_cast<char*>(&n), 8);
+    if (!f || n > (1u << 28)) throw std::runtime_error(path + ": no safetensors header");
+    std::string head((size_t)n, ' ');
+    f.read(&head[0], (std::streamsize)n);
+    if (!f) throw std::runtime_error(path + ": header length exceeds the file");
+    return JsonReader(head).parse();
+}
+
+// config.json of a layered design -> layer descriptors (the keys zig_gpt2_amd/lm.py reads).  tensors: the checkpoint's
+// safetensors header, for the sizes that only a tensor's shape gives (may be null when the configuration lists them).
+inline void build_config(const Json& cfg, const Json* tensors, std::vector<zg_lm_layer>& layers, zg_lm_config& out) {
     const Json* arch = cfg.get("architecture");
-    if (!arch || arch->str != "Tokosun") throw std::runtime_error("config: architecture '" + (arch ? arch->str : std::string("?")) + "' is not served");
+    const std::string design = arch ? arch->str : std::string("?");
+    if (design != "Tokosun" && design != "Gupizen") throw std::runtime_error("config: architecture '" + design + "' is not served");
+    const bool gup = design == "Gupizen";
     memset(&out, 0, sizeof(out));
+    if (gup) {  // what the name fixes: tied head, the embedding output added again per repetition of the loop
+        out.flags |= ZG_LM_TIED_HEAD | ZG_LM_LOOP_READD;
+        out.embed_scale = 1.0f;
+        if (const Json* e = cfg.get("embedding"))
+            if (e->truthy())
+                if (const Json* v = e->get("scale")) out.embed_scale = (float)v->num;
+        if (const Json* c = cfg.get("canon"))
+            if (c->truthy())
+                if (const Json* v = c->get("taps")) out.canon_taps = (int)v->num;
+    }
+    size_t layer_index = 0;
     out.vocab = (size_t)cfg.at("vocab").num;
     out.width = (size_t)cfg.at("width").num;
     out.norm_eps = (float)cfg.at("norm").at("eps").num;
@@ -160,10 +187,54 @@ inline void build_config(const Json& cfg, std::vector<zg_lm_layer>& layers, zg_l
         memset(&d, 0, sizeof(d));
         const std::string& type = e.at("type").str;
         const Json& m = e.at("mixer");
-        d.heads = (int)m.at("heads").num;
-        d.dim = (int)m.at("dim").num;
-        d.vdim = (int)m.at("vdim").num;
-        if (type == "hgrn2") {
+        const std::string prefix = "l" + std::to_string(layer_index++) + ".";
+        const Json& sizes = (gup && type == "parallel") ? m.at("left") : m;
+        d.heads = (int)sizes.at("heads").num;
+        d.dim = (int)sizes.at("dim").num;
+        d.vdim = (int)sizes.at("vdim").num;
+        if (gup) {
+            d.ff_act = ZG_LM_ACT_GELU;
+            d.router = ZG_LM_ROUTE_TOP_LOGITS;
+            d.kv_heads = sizes.get("kv_heads") ? (int)sizes.at("kv_heads").num : d.heads;
+        }
+        if (gup && type == "parallel") {
+            d.mixer = ZG_LM_MIX_PARALLEL;
+            d.scale = (float)sizes.at("scale").num;
+            if (const Json* mask = sizes.get("mask"))
+                if (mask->truthy())
+                    if (const Json* v = mask->get("size")) d.window = (int)v->num;
+            d.rot_base = 10000.0f;
+            if (const Json* rot = sizes.get("rot"))
+                if (rot->truthy()) {
+                    if (const Json* v = rot->get("dims")) d.rot_dims = (int)v->num;
+                    if (const Json* v = rot->get("base")) d.rot_base = (float)v->num;
+                    const Json* sc = rot->get("scaling");
+                    if (sc && sc->truthy()) {  // wavelength bands: `high` / `low` travel in the fields of the blend's `fast` / `slow`
+                        d.rot_scaled = ZG_LM_ROT_BANDS;
+                        d.rot_factor = (float)sc->at("factor").num;
+                        d.rot_original = (float)sc->at("original").num;
+                        d.rot_fast = (float)sc->at("high").num;
+                        d.rot_slow = (float)sc->at("low").num;
+                    }
+                }
+            const Json& r = m.at("right");
+            d.lru_width = (int)r.at("width").num;
+            d.lru_blocks = (int)r.at("blocks").num;
+            d.lru_conv = (int)r.at("conv").num;
+        } else if (gup && type == "channel_delta") {
+            d.mixer = ZG_LM_MIX_CHANNEL_DELTA;
+            d.conv = (int)m.at("conv").num;
+            auto inner = [&](const char* key, const char* tensor) -> int {
+                if (const Json* v = m.get(key)) return (int)v->num;
+                const Json* t = tensors ? tensors->get(prefix + tensor) : nullptr;
+                if (!t) throw std::runtime_error("config: the inner size '" + std::string(key) + "' needs the shape of tensor " + prefix + tensor);
+                return (int)t->at("shape").arr.at(0).num;
+            };
+            d.decay_rank = inner("decay_rank", "mix.a1");
+            d.gate_rank = inner("gate_rank", "mix.g1");
+        } else if (gup) {
+            throw std::runtime_error("config: unknown mixer type '" + type + "'");
+        } else if (type == "hgrn2") {
             d.mixer = ZG_LM_MIX_HGRN2;
         } else if (type == "latent_attention") {
             d.mixer = ZG_LM_MIX_LATENT_ATTENTION;
@@ -306,12 +377,13 @@ inline int lm_main(int argc, char** argv) {
         }
         std::vector<zg_lm_layer> layers;
         zg_lm_config cfg;
-        build_config(JsonReader(slurp(dir + "/config.json")).parse(), layers, cfg);
+        const Json tensors = safetensors_header(dir + "/model.safetensors");
+        build_config(JsonReader(slurp(dir + "/config.json")).parse(), &tensors, layers, cfg);
         size_t longest = 0, stride = 0;
         for (auto& pr : prompts) longest = std::max(longest, pr.size() + n_new), stride = std::max(stride, pr.size());
         cfg.max_seqs = prompts.size();
         cfg.max_tokens = prompts.size() * (longest + 64);
-        cfg.flags = flags;
+        cfg.flags |= flags;
         zg_lm* g = nullptr;
         if (zg_lm_create(&g, &cfg, 0) != ZG_OK) throw std::runtime_error(std::string("create: ") + zg_last_error());
         load_safetensors(g, dir + "/model.safetensors");
