@@ -48,6 +48,9 @@ def parse():
                    help="instead of the default workload: prompt and decode throughput of a layered model (Tokosun design, random weights) "
                         "at a size that resembles GPT-2 124M / medium / XL, beside the GPT-2 model of the same width and depth")
     p.add_argument("--lm-dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    p.add_argument("--lm-design", default="tokosun", choices=["tokosun", "gupizen"],
+                   help="with --lm: which design is measured.  gupizen: a Gupizen stack of the same width and depth, beside the Tokosun stack "
+                        "(the tier's closest model) instead of GPT-2")
     p.add_argument("--dry-run", action="store_true",
                    help="CPU rehearsal of the launch path (gloo, no GPU, no kernels): rendezvous, prompt sharding, "
                         "weight-arena broadcast, barriers and the max-reduce; prints a line with dry_run=true")
@@ -441,6 +444,25 @@ def lm_bench_config(width, n_layers, vocab):
     return lm.LMConfig(vocab=vocab, width=width, layers=[lm.LayerSpec(**order[i % 4]) for i in range(n_layers)], norm_eps=1e-6)
 
 
+def gupizen_bench_config(width, n_layers, vocab, window=512):
+    """A Gupizen-design stack of `n_layers` layers in the repeating order parallel, delta rule, parallel, parallel, every layer with
+    8 plain experts of width `width` of which 2 are chosen: attention heads of 64 channels on a quarter as many key heads, a window
+    of 512 tokens, a recurrent unit as wide as the model, delta-rule heads of 128 x 128, input convolutions of 4 taps."""
+    from zig_gpt2_amd import lm
+
+    heads = width // 64
+    kv = heads // 4 if heads % 4 == 0 else heads // 5 if heads % 5 == 0 else heads
+    moe = dict(ff="moe", ff_width=width, experts=8, top=2, expert_act="gelu", router="top_logits")
+    par = dict(mixer="parallel", heads=heads, kv_heads=kv, dim=64, vdim=64, scale=64 ** -0.5, window=window, rot_dims=32, rot_base=10000.0,
+               rot_scaling={"factor": 4.0, "original": 2048, "low": 1.0, "high": 4.0}, rot_style="bands", lru_width=width, lru_blocks=heads,
+               lru_conv=4, **moe)
+    hd = 128 if width % 128 == 0 else 64
+    dl = dict(mixer="channel_delta", heads=width // hd, kv_heads=width // hd, dim=hd, vdim=hd, conv=4, decay_rank=64, gate_rank=64, **moe)
+    order = [par, dl, par, par]
+    return lm.LMConfig(vocab=vocab, width=width, layers=[lm.LayerSpec(**order[i % 4]) for i in range(n_layers)], norm_eps=1e-6,
+                       architecture="Gupizen", embed_scale=1.0, canon_taps=4)
+
+
 def lm_weight_bytes(cfg):
     """(stored, read per decoded token) bytes of the bf16 matrices: every expert is stored, `top` of them are read."""
     stored = active = 0
@@ -465,15 +487,21 @@ def lm_bench(a):
     gname, width, n_layers = LM_SIZES[a.lm]
     gcfg = synth.CONFIGS.get(gname) or synth.GPTConfig(50257, 1024, n_layers, width // 64, width)
     ctx = a.ctx or 1024
+    gup = a.lm_design == "gupizen"
     cfg = lm_bench_config(width, n_layers, gcfg.vocab_size)
     out = {"metric": "lm_decode_tokens_per_s", "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "higher_is_better": True,
            "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if a.lm_dtype == "bfloat16" else "fp32", "data": "synthetic (random weights, filled on the GPU)",
            "config": {"model": f"Tokosun design, width {width}, {n_layers} layers (recurrence+dense, attention+experts x2, recurrence+experts), vocab {gcfg.vocab_size}",
                       "global_batch": 1, "seq_len": ctx, "parallelism": "single GPU"}}
-    m = lm.LayeredLM(cfg, dtype=a.lm_dtype, max_tokens=8 * ctx + 64, max_seqs=8, max_step_tokens=8 * ctx)
-    m.init_random(seed=a.seed + 1, std=0.02)
-    stored, active = lm_weight_bytes(cfg)
     rng = np.random.default_rng(a.seed)
+    m = cfg = stored = active = None
+
+    def open_model(c):
+        nonlocal m, cfg, stored, active
+        cfg = c
+        m = lm.LayeredLM(cfg, dtype=a.lm_dtype, max_tokens=8 * ctx + 64, max_seqs=8, max_step_tokens=8 * ctx)
+        m.init_random(seed=a.seed + 1, std=0.02)
+        stored, active = lm_weight_bytes(cfg)
 
     def prompt_pass(n_prompts, n):
         toks = [rng.integers(0, cfg.vocab, n).astype(np.int32) for _ in range(n_prompts)]
@@ -505,9 +533,23 @@ def lm_bench(a):
         best["frac_of_8TBps_weights_only"] = round(active / (best["device_us_per_step"] * 1e-6) / 1e9 / HBM_PEAK_GBS, 4) if n_prompts == 1 else None
         return best
 
-    lm_res = {"weights_bytes_stored": stored, "weights_bytes_read_per_token": active,
-              "prefill": [prompt_pass(1, ctx - 1), prompt_pass(8, ctx - 1), prompt_pass(1, 128)], "decode": [decode(1), decode(8)]}
-    m.close()
+    def measure(c):
+        open_model(c)
+        res = {"weights_bytes_stored": stored, "weights_bytes_read_per_token": active,
+               "prefill": [prompt_pass(1, ctx - 1), prompt_pass(8, ctx - 1), prompt_pass(1, 128)], "decode": [decode(1), decode(8)]}
+        m.close()
+        return res
+
+    if gup:  # the new design beside the tier's closest model at equal width and depth
+        g_res = measure(gupizen_bench_config(width, n_layers, gcfg.vocab_size))
+        t_res = measure(lm_bench_config(width, n_layers, gcfg.vocab_size))
+        d1 = g_res["decode"][0]
+        out["config"]["model"] = (f"Gupizen design, width {width}, {n_layers} layers (parallel, delta rule, parallel, parallel; 8 experts, 2 chosen; "
+                                  f"window 512), vocab {gcfg.vocab_size}")
+        out.update(value=d1["tokens_per_s"], ms_per_step=round(d1["wall_us_per_step"] / 1e3, 4), gupizen=g_res, tokosun_equal_size=t_res)
+        print(json.dumps(out))
+        return
+    lm_res = measure(lm_bench_config(width, n_layers, gcfg.vocab_size))
 
     # GPT-2 of the same width and depth through its own tier (captured decode graphs, whole-prompt pass)
     lib = _lib.load()

@@ -190,6 +190,21 @@ def test_slots_and_pages_are_reused():
     m.close()
 
 
+def test_general_window_kernel(monkeypatch):
+    """The one-workgroup-per-row form of the windowed attention (what a step takes when the split form's workspace would not
+    fit), on prompts, portions and decoded tokens, windows of several key tiles included."""
+    monkeypatch.setenv("ZGPT2_LM_WINDOW_GENERAL", "1")
+    cfg = gl.config([gl.parallel_layer(window=0), gl.parallel_layer(heads=2, kv_heads=1, dim=70, vdim=6, window=90, rot_dims=30)])
+    w = gl.weights(cfg, seed=21)
+    toks = gl.tokens(22, 200, cfg["vocab"])
+    ref = go.Model(cfg, w).forward(toks)[0]
+    for dtype in ("float32", "bfloat16"):
+        m = make(cfg, w, dtype)
+        tl.assert_close(run_whole(m, toks), ref, dtype)
+        tl.assert_close(run_cut(m, toks, [3, 64, 65, 130] + list(range(180, 200))), ref, dtype)
+        m.close()
+
+
 def _edge_model(window, n, seed):
     """One parallel layer whose attention is sharp (large score factor, no rotary on the scores' channels beyond two): most
     queries put nearly all their weight on one key.  Returns (cfg, weights, oracle, distance of the heaviest key per head and query)."""

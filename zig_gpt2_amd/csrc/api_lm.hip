@@ -176,7 +176,8 @@ struct zg_lm {
     float *gu_buf = nullptr, *hb = nullptr, *ye = nullptr, *wt = nullptr, *last_h = nullptr, *hn = nullptr, *logits = nullptr;
     float *row_max = nullptr, *samp_ws = nullptr, *samp_u = nullptr, *amax_val = nullptr;
     int* amax_idx = nullptr;
-    float *attn_ws = nullptr, *scan_ws = nullptr;
+    float *attn_ws = nullptr, *scan_ws = nullptr, *win_ws = nullptr;
+    size_t win_ws_floats = 0;
     float *x0 = nullptr, *hc = nullptr, *y2 = nullptr, *ta = nullptr, *tb = nullptr, *tc = nullptr, *td = nullptr;
     size_t scan_ws_floats = 0;
     size_t attn_ws_floats = 0;
@@ -241,7 +242,7 @@ void layout(zg_lm* g, Bump& b) {
         mat("head", g->head, 0, V, W);
     }
     vec("final.norm", g->final_norm, W, INIT_OFFSET);
-    size_t max_t = 1;
+    size_t max_t = 1, max_win = 0;
     size_t max_proj = 1, max_qr = 1, max_q = 1, max_qa = 1, max_ctx = 1, max_o = 1, max_ff = 1, max_assign = 1, max_gu = 1, max_hb = 1, max_e = 1, max_att_part = 0, max_scan = 0;
     for (size_t i = 0; i < g->layers.size(); ++i) {
         LayerW& L = g->layers[i];
@@ -286,6 +287,7 @@ void layout(zg_lm* g, Bump& b) {
             max_proj = std::max(max_proj, NP);
             max_o = std::max(max_o, HV);
             max_t = std::max(max_t, C);
+            max_win = std::max(max_win, window_split_workspace((int)MS, (int)H, (int)Vd, d.window > 0 ? d.window : g->max_pages * g->P, nullptr));
         } else if (d.mixer == ZG_LM_MIX_CHANNEL_DELTA) {
             const size_t G = d.kv_heads, HV = H * Vd, CC = 2 * G * D + HV, RA = d.decay_rank, RG = d.gate_rank;
             const size_t NP = CC + H + RA + RG;
@@ -454,6 +456,12 @@ void layout(zg_lm* g, Bump& b) {
     g->scan_ws = b.take<float>(std::max<size_t>(1, g->scan_ws_floats));
     g->attn_ws_floats = (size_t)kGemvMaxRows * kAttnSplits * max_att_part;
     g->attn_ws = b.take<float>(std::max<size_t>(1, g->attn_ws_floats));
+    // scores and partial sums of the split windowed attention: up to 2 GiB for a whole portion, else for steps of few rows only
+    // (longer steps of such a model then take the general kernel)
+    if (max_win > ((size_t)1 << 29)) max_win = max_win / MS * kGemvMaxRows;
+    if (max_win > ((size_t)1 << 29)) max_win = 0;
+    g->win_ws_floats = max_win;
+    g->win_ws = b.take<float>(std::max<size_t>(1, max_win));
     g->last_h = b.take<float>((size_t)g->n_passes * NS * W);
     g->hn = b.take<float>((size_t)g->logit_rows * W);
     g->logits = b.take<float>((size_t)g->logit_rows * V);
@@ -602,8 +610,13 @@ int enqueue_layers(zg_lm* g, int M, int n_ent, bool capturing, bool single) {
             ZG_TRY(launch_linear(lin, f32, s));
             // left: attention inside the window
             ZG_TRY(launch_window_prep(g->proj, NP, M, H, G, D, Vd, rot, L.vfreq, d_pos, d_slot, g->page_table, g->max_pages, g->P, ps.cache, s));
-            ZG_TRY(launch_window_attention(g->proj, NP, g->o, HV, M, H, G, D, Vd, d.scale, d.window, L.sink, L.talk, L.vfreq, d_pos, d_slot,
-                                           g->page_table, g->max_pages, g->P, ps.cache, s));
+            bool split = false;
+            ZG_TRY(launch_window_attention_split(g->proj, NP, g->o, HV, M, H, G, D, Vd, d.scale, d.window, L.sink, L.talk, L.vfreq, d_pos, d_slot,
+                                                 g->page_table, g->max_pages, g->P, ps.cache, d.window > 0 ? d.window : g->max_pages * g->P, g->win_ws,
+                                                 g->win_ws_floats, s, &split));
+            if (!split)
+                ZG_TRY(launch_window_attention(g->proj, NP, g->o, HV, M, H, G, D, Vd, d.scale, d.window, L.sink, L.talk, L.vfreq, d_pos, d_slot,
+                                               g->page_table, g->max_pages, g->P, ps.cache, s));
             lin = Linear();
             lin.A = g->o; lin.lda = HV; lin.B = L.o; lin.ldb = HV; lin.C = g->y; lin.ldc = W; lin.M = M; lin.N = W; lin.K = HV;
             ZG_TRY(launch_linear(lin, f32, s));

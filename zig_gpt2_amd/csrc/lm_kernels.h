@@ -149,6 +149,17 @@ int launch_window_attention(const float* q, int ldq, float* out, int ldo, int M,
                             const float* sink, const float* talk, const float* vfreq, const int* row_pos, const int* row_slot,
                             const int* page_table, int max_pages, int page_tokens, const float* cache, hipStream_t s);
 
+// The same with a row's keys split over up to kWinSplits workgroups and the scores kept in a workspace (three launches): what
+// steps of few rows need to fill the chip, and prompt portions to compute every score once.  key_capacity: the most keys a row
+// can see (the window, or the longest sequence).  ws: window_split_workspace(rows, ...) floats.  *taken = false (nothing
+// launched) when the workspace is too small or a size is beyond the kernels' limits.
+constexpr int kWinSplits = 16;
+size_t window_split_workspace(int rows, int H, int V, int key_capacity, int* n_split_out);
+int launch_window_attention_split(const float* q, int ldq, float* out, int ldo, int M, int H, int G, int D, int V, float scale, int window,
+                                  const float* sink, const float* talk, const float* vfreq, const int* row_pos, const int* row_slot,
+                                  const int* page_table, int max_pages, int page_tokens, const float* cache, int key_capacity, float* ws,
+                                  size_t ws_floats, hipStream_t s, bool* taken);
+
 // ------------------------------------------------------------------------------------------------ real-gated linear recurrent unit
 // Per entry and channel c: r = sigmoid(gr + br), i = sigmoid(gi + bi), a = exp(-8 r softplus(lam)), S = a S + sqrt(1 - a^2) i u,
 // out = S * gelu_tanh(y + by); S = state[slot][c], read at the start of the entry and written back at its end.

@@ -7,6 +7,7 @@
 //   * the gated delta rule with one decay per key channel (a matrix state per head).
 // Everything here is fp32 in both precision modes: positions, angles, scores, weights, gates, decays, recurrent states.
 #include <math.h>
+#include <stdlib.h>
 
 #include <algorithm>
 
@@ -249,42 +250,235 @@ __global__ __launch_bounds__(256) void window_attention_kernel(const float* q, i
     }
 }
 
-// ------------------------------------------------------------------------------------------------ gated linear recurrent unit
-// Per entry and channel, token by token:  r = sigmoid(gr + br), i = sigmoid(gi + bi), a = exp(-8 r softplus(lam)),
-// S = a S + sqrt(1 - a^2) i u,  out = S * gelu_tanh(y + by).  The loads of a token do not depend on S: eight tokens are
-// requested together.
-__global__ __launch_bounds__(64) void rglru_scan_kernel(const float* u, int ldu, const float* gr, const float* gi, int ldg, const float* br,
-                                                        const float* bi, const float* lam, const float* y, int ldy, const float* by,
-                                                        float* out, int ldo, int C, float* state, size_t slot_stride, const int* ent_start,
-                                                        const int* ent_len, const int* ent_slot) {
-    const int e = blockIdx.x, c = blockIdx.y * blockDim.x + threadIdx.x;
-    if (c >= C) return;
-    const int n = ent_len[e], m0 = ent_start[e];
-    if (n <= 0) return;
-    float* sp = state + (size_t)ent_slot[e] * slot_stride + c;
-    float S = *sp;
-    const float sl = softplus_f(lam[c]), brc = br[c], bic = bi[c], byc = by[c];
-    for (int t0 = 0; t0 < n; t0 += 8) {
-        float uu[8], rr[8], ii[8], yy[8];
+// The same attention with a row's keys split over several workgroups, in three launches (scores and weights pass through a
+// workspace, so no score is computed twice and a one-row step still fills many compute units):
+//   scores   workgroup (split, row): s_h(j) for its share of the row's keys — a wave per key, lanes over the D channels, one
+//            wave reduction per head — written to sc[row][h][j - first key]; per head the share's maximum and sum of exp
+//   mix      workgroup (split, row): the row's maximum and denominator per head from all shares (and the sink), then for its
+//            keys the normalised weights, their mix over the heads, and the share's weighted sum of values
+//   merge    workgroup (row): the shares' sums added in split order, turned back by the row's position
+// A share is ceil(keys of the row / splits) consecutive keys: the order of every sum depends on the position alone.
+constexpr int kMixTile = 32;
+
+__device__ __forceinline__ void window_range(int pos, int window, int n_split, int split, int& j_lo, int& k0, int& k1) {
+    j_lo = window > 0 ? max(0, pos - window + 1) : 0;
+    const int n_keys = pos - j_lo + 1, chunk = (n_keys + n_split - 1) / n_split;
+    k0 = min(n_keys, split * chunk);
+    k1 = min(n_keys, k0 + chunk);
+}
+
+template <int RPL>
+__global__ __launch_bounds__(256) void window_scores_kernel(const float* q, int ldq, int H, int G, int D, int V, float scale, int window,
+                                                            const int* row_pos, const int* row_slot, const int* page_table, int max_pages,
+                                                            int page_tokens, const float* cache, float* sc, int NK, float* st) {
+    extern __shared__ __attribute__((aligned(16))) float s_sc[];
+    float* s_q = s_sc;           // [H][64 RPL] (zero beyond D)
+    float* s_m = s_q + H * 64 * RPL;  // [4][H]
+    float* s_l = s_m + 4 * H;         // [4][H]
+    const int split = blockIdx.x, n_split = gridDim.x, m = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int pos = row_pos[m];
+    int j_lo, k0, k1;
+    window_range(pos, window, n_split, split, j_lo, k0, k1);
+    const int* pages = page_table + (size_t)row_slot[m] * max_pages;
+    const int rep = H / G;
+    const size_t cstride = (size_t)G * (D + V);
+    for (int i = threadIdx.x; i < H * 64 * RPL; i += blockDim.x) {
+        const int h = i / (64 * RPL), d = i % (64 * RPL);
+        s_q[i] = d < D ? q[(size_t)m * ldq + (size_t)h * D + d] : 0.0f;
+    }
+    for (int i = threadIdx.x; i < 4 * H; i += blockDim.x) {
+        s_m[i] = -INFINITY;
+        s_l[i] = 0.0f;
+    }
+    __syncthreads();
+    float* srow = sc + (size_t)m * H * NK;
+    for (int kk = k0 + wave; kk < k1; kk += 4) {
+        const int j = j_lo + kk;
+        const float* kr = cache + ((size_t)pages[(j / page_tokens) % max_pages] * page_tokens + j % page_tokens) * cstride;
+        for (int g = 0; g < G; ++g) {
+            float kd[RPL];
 #pragma unroll
-        for (int k = 0; k < 8; ++k) {
-            const bool ok = t0 + k < n;
-            const size_t m = (size_t)(m0 + t0 + k);
-            uu[k] = ok ? u[m * ldu + c] : 0.0f;
-            rr[k] = ok ? gr[m * ldg + c] : 0.0f;
-            ii[k] = ok ? gi[m * ldg + c] : 0.0f;
-            yy[k] = ok ? y[m * ldy + c] : 0.0f;
-        }
+            for (int r = 0; r < RPL; ++r) kd[r] = lane + 64 * r < D ? kr[(size_t)g * D + lane + 64 * r] : 0.0f;
+            for (int hh = 0; hh < rep; ++hh) {
+                const int h = g * rep + hh;
+                float a = 0.0f;
 #pragma unroll
-        for (int k = 0; k < 8; ++k) {
-            if (t0 + k < n) {
-                const float a = expf(-8.0f * sigmoid_f(rr[k] + brc) * sl);
-                S = fmaf(a, S, sqrtf(1.0f - a * a) * sigmoid_f(ii[k] + bic) * uu[k]);
-                out[(size_t)(m0 + t0 + k) * ldo + c] = S * gelu_tanh_f(yy[k] + byc);
+                for (int r = 0; r < RPL; ++r) a = fmaf(s_q[h * 64 * RPL + lane + 64 * r], kd[r], a);
+                a = wave_allsum(a) * scale;
+                if (lane == 0) {
+                    srow[(size_t)h * NK + kk] = a;
+                    const float mo = s_m[wave * H + h], mn = fmaxf(mo, a);
+                    s_l[wave * H + h] = s_l[wave * H + h] * expf(mo - mn) + expf(a - mn);
+                    s_m[wave * H + h] = mn;
+                }
             }
         }
     }
-    *sp = S;
+    __syncthreads();
+    for (int h = threadIdx.x; h < H; h += blockDim.x) {
+        float mx = -INFINITY;
+        for (int w = 0; w < 4; ++w) mx = fmaxf(mx, s_m[w * H + h]);
+        float l = 0.0f;
+        for (int w = 0; w < 4; ++w) l += s_l[w * H + h] > 0.0f ? s_l[w * H + h] * expf(s_m[w * H + h] - mx) : 0.0f;
+        float* o = st + (((size_t)m * n_split + split) * H + h) * 2;
+        o[0] = mx;
+        o[1] = l;
+    }
+}
+
+__global__ __launch_bounds__(256) void window_mix_kernel(int H, int G, int D, int V, int window, const float* sink, const float* talk,
+                                                         const int* row_pos, const int* row_slot, const int* page_table, int max_pages,
+                                                         int page_tokens, const float* cache, const float* sc, int NK, const float* st,
+                                                         float* po) {
+    extern __shared__ __attribute__((aligned(16))) float s_mx[];
+    float* s_p = s_mx;                  // [H][kMixTile]
+    float* s_w = s_p + H * kMixTile;    // [H][kMixTile]
+    float* s_talk = s_w + H * kMixTile; // [H H]
+    float* s_M = s_talk + H * H;        // [H]
+    float* s_iZ = s_M + H;              // [H]
+    __shared__ int s_row[kMixTile];
+    const int split = blockIdx.x, n_split = gridDim.x, m = blockIdx.y, tid = threadIdx.x;
+    const int pos = row_pos[m];
+    int j_lo, k0, k1;
+    window_range(pos, window, n_split, split, j_lo, k0, k1);
+    const int* pages = page_table + (size_t)row_slot[m] * max_pages;
+    const int rep = H / G;
+    const size_t cstride = (size_t)G * (D + V);
+    for (int i = tid; i < H * H; i += blockDim.x) s_talk[i] = talk ? talk[i] : ((i / H) == (i % H) ? 1.0f : 0.0f);
+    for (int h = tid; h < H; h += blockDim.x) {
+        const float* sp = st + ((size_t)m * n_split * H + h) * 2;
+        float mx = sink ? sink[h] : -INFINITY;
+        for (int s2 = 0; s2 < n_split; ++s2) mx = fmaxf(mx, sp[(size_t)s2 * H * 2]);
+        float z = sink ? expf(sink[h] - mx) : 0.0f;
+        for (int s2 = 0; s2 < n_split; ++s2) {
+            const float l = sp[(size_t)s2 * H * 2 + 1];
+            if (l > 0.0f) z += l * expf(sp[(size_t)s2 * H * 2] - mx);
+        }
+        s_M[h] = mx;
+        s_iZ[h] = 1.0f / z;
+    }
+    float acc[kWinAcc];
+#pragma unroll
+    for (int r = 0; r < kWinAcc; ++r) acc[r] = 0.0f;
+    const float* srow = sc + (size_t)m * H * NK;
+    for (int t0 = k0; t0 < k1; t0 += kMixTile) {
+        const int nt = min(kMixTile, k1 - t0);
+        __syncthreads();
+        if (tid < nt) {
+            const int j = j_lo + t0 + tid;
+            s_row[tid] = pages[(j / page_tokens) % max_pages] * page_tokens + j % page_tokens;
+        }
+        for (int idx = tid; idx < H * kMixTile; idx += blockDim.x) {
+            const int h = idx / kMixTile, jj = idx % kMixTile;
+            s_p[idx] = jj < nt ? expf(srow[(size_t)h * NK + t0 + jj] - s_M[h]) * s_iZ[h] : 0.0f;
+        }
+        __syncthreads();
+        for (int idx = tid; idx < H * kMixTile; idx += blockDim.x) {
+            const int h = idx / kMixTile, jj = idx % kMixTile;
+            float wsum = 0.0f;
+            for (int g = 0; g < H; ++g) wsum = fmaf(s_talk[h * H + g], s_p[g * kMixTile + jj], wsum);
+            s_w[idx] = wsum;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < kWinAcc; ++r) {
+            const int o = tid + 256 * r;
+            if (o < H * V) {
+                const int h = o / V, c = o % V;
+                const float* vbase = cache + (size_t)G * D + (size_t)(h / rep) * V + c;
+                float a = acc[r];
+                for (int jj = 0; jj < nt; ++jj) a = fmaf(s_w[h * kMixTile + jj], vbase[(size_t)s_row[jj] * cstride], a);
+                acc[r] = a;
+            }
+        }
+    }
+    float* orow = po + ((size_t)m * n_split + split) * H * V;
+#pragma unroll
+    for (int r = 0; r < kWinAcc; ++r) {
+        const int o = tid + 256 * r;
+        if (o < H * V) orow[o] = acc[r];
+    }
+}
+
+__global__ __launch_bounds__(256) void window_merge_kernel(const float* po, int n_split, float* out, int ldo, int H, int V, const float* vfreq,
+                                                           const int* row_pos) {
+    const int m = blockIdx.x;
+    const float fpos = (float)row_pos[m];
+    const float* base = po + (size_t)m * n_split * H * V;
+    for (int p = threadIdx.x; p < H * V / 2; p += blockDim.x) {  // a pair of channels: (2i, 2i + 1) of a head
+        float a = 0.0f, b = 0.0f;
+        for (int s2 = 0; s2 < n_split; ++s2) {
+            a += base[(size_t)s2 * H * V + 2 * p];
+            b += base[(size_t)s2 * H * V + 2 * p + 1];
+        }
+        float sn, cs;
+        sincosf(fpos * vfreq[p % (V / 2)], &sn, &cs);
+        out[(size_t)m * ldo + 2 * p] = a * cs + b * sn;
+        out[(size_t)m * ldo + 2 * p + 1] = b * cs - a * sn;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------ gated linear recurrent unit
+// Per entry and channel:  r = sigmoid(gr + br), i = sigmoid(gi + bi), a = exp(-8 r softplus(lam)),
+// S = a S + sqrt(1 - a^2) i u,  out = S * gelu_tanh(y + by).  The recurrence is linear in S, so an entry's tokens are cut into
+// kLruSegs stretches that run side by side: every stretch from a zero state (its end value and the product of its a), the
+// start states down the stretches (one thread per channel), every stretch again from its true start, writing the outputs.
+// A workgroup is 64 channels x kLruSegs stretches.  Entries of few tokens take one stretch, once.
+constexpr int kLruSegs = 16;
+__global__ __launch_bounds__(64 * kLruSegs) void rglru_scan_kernel(const float* u, int ldu, const float* gr, const float* gi, int ldg,
+                                                                   const float* br, const float* bi, const float* lam, const float* y, int ldy,
+                                                                   const float* by, float* out, int ldo, int C, float* state,
+                                                                   size_t slot_stride, const int* ent_start, const int* ent_len,
+                                                                   const int* ent_slot) {
+    __shared__ float s_a[kLruSegs][64], s_b[kLruSegs][64];
+    const int e = blockIdx.x, cl = threadIdx.x & 63, seg = threadIdx.x >> 6, c = blockIdx.y * 64 + cl;
+    const int n = ent_len[e], m0 = ent_start[e];
+    if (n <= 0) return;
+    const bool ok = c < C;
+    const int cc = ok ? c : 0;
+    const bool cut = n >= 4 * kLruSegs;
+    const int len = cut ? (n + kLruSegs - 1) / kLruSegs : n;
+    const int t_lo = min(n, seg * len), t_hi = cut ? min(n, t_lo + len) : (seg == 0 ? n : 0);
+    float* sp = state + (size_t)ent_slot[e] * slot_stride + cc;
+    const float sl = softplus_f(lam[cc]), brc = br[cc], bic = bi[cc], byc = by[cc];
+    auto coef = [&](int t, float& a, float& b) {
+        const size_t m = (size_t)(m0 + t);
+        a = expf(-8.0f * sigmoid_f(gr[m * ldg + cc] + brc) * sl);
+        b = sqrtf(1.0f - a * a) * sigmoid_f(gi[m * ldg + cc] + bic) * u[m * ldu + cc];
+    };
+    float S = 0.0f;
+    if (cut) {
+        float A = 1.0f;
+        for (int t = t_lo; t < t_hi; ++t) {
+            float a, b;
+            coef(t, a, b);
+            S = fmaf(a, S, b);
+            A *= a;
+        }
+        s_a[seg][cl] = A;
+        s_b[seg][cl] = S;
+        __syncthreads();
+        if (seg == 0) {  // start state of every stretch, in place of its end value
+            float run = *sp;
+            for (int g2 = 0; g2 < kLruSegs; ++g2) {
+                const float next = fmaf(s_a[g2][cl], run, s_b[g2][cl]);
+                s_b[g2][cl] = run;
+                run = next;
+            }
+            if (ok) *sp = run;
+        }
+        __syncthreads();
+        S = s_b[seg][cl];
+    } else {
+        S = *sp;
+    }
+    for (int t = t_lo; t < t_hi; ++t) {
+        float a, b;
+        coef(t, a, b);
+        S = fmaf(a, S, b);
+        if (ok) out[(size_t)(m0 + t) * ldo + c] = S * gelu_tanh_f(y[(size_t)(m0 + t) * ldy + c] + byc);
+    }
+    if (!cut && seg == 0 && ok) *sp = S;
 }
 
 // y = (l / rms(l) * wl + r / rms(r) * wr) / 2, rows of W floats
@@ -325,101 +519,101 @@ __global__ __launch_bounds__(256) void delta_prep_kernel(float* qk, int ldqk, in
     }
 }
 
-// One workgroup per (entry, head); the head's state S[D][V] sits in registers: thread (rg, c) holds rows rg, rg + NR, ... of
-// column c (NR = 256 / VP row groups, VP = the power of two >= V).  Token by token:
-//   S <- g S (rows);  kv = S^T k;  u = beta (v - kv);  S <- S + k u^T;  o = S^T q
-// The two column sums meet in the LDS; the token's vectors are fetched one token ahead.
-template <int RPT>
+// The recurrence of a head runs column by column of its state: u_c = beta (v_c - S[:, c] . k), S[:, c] += k u_c,
+// o_c = S[:, c] . q touch no other column.  A wave owns kDeltaCols columns, its lanes split the D rows (RPL rows a lane), so both
+// column sums are wave reductions and a token needs no barrier; a workgroup's four waves take neighbouring columns and the
+// grid covers (entry, head, column group): many more waves than heads.  Every wave reads the token's q, k and decay itself (one
+// coalesced load per vector, shared through the caches), one token ahead of its use.
+constexpr int kDeltaCols = 4;
+template <int RPL>
 __global__ __launch_bounds__(256) void delta_scan_kernel(const float* qk, int ldqk, const float* v, int ldv, const float* beta, int ldb,
-                                                         const float* dec, int ldd, float* out, int ldo, int H, int G, int D, int V, int VP,
+                                                         const float* dec, int ldd, float* out, int ldo, int H, int G, int D, int V,
                                                          float* state, size_t slot_stride, const int* ent_start, const int* ent_len,
                                                          const int* ent_slot) {
-    extern __shared__ __attribute__((aligned(16))) float s_delta[];
-    const int NR = 256 / VP;
-    const int n_stage = 3 * D + V + 1;      // q | k | g | v | beta
-    float* s_stage = s_delta;               // [2][n_stage]
-    float* s_p1 = s_stage + 2 * n_stage;    // [NR][VP]
-    float* s_p2 = s_p1 + NR * VP;           // [NR][VP]
-    const int e = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+    const int e = blockIdx.x, h = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int c0 = (blockIdx.z * 4 + wave) * kDeltaCols;
     const int n = ent_len[e], m0 = ent_start[e];
-    if (n <= 0) return;
-    const int c = tid % VP, rg = tid / VP, kvh = h / (H / G);
-    const bool col_ok = c < V;
+    if (n <= 0 || c0 >= V) return;
+    const int kvh = h / (H / G);
     float* Sg = state + (size_t)ent_slot[e] * slot_stride + (size_t)h * D * V;
-    float S[RPT];
+    float S[kDeltaCols][RPL];
 #pragma unroll
-    for (int r = 0; r < RPT; ++r) {
-        const int d = rg + NR * r;
-        S[r] = (col_ok && d < D) ? Sg[(size_t)d * V + c] : 0.0f;
-    }
-    constexpr int kPre = 5;  // 256 * 5 >= 3 * 256 + 256 + 1
-    auto fetch = [&](int t, float pre[kPre]) {
+    for (int c = 0; c < kDeltaCols; ++c)
+#pragma unroll
+        for (int r = 0; r < RPL; ++r) {
+            const int d = lane + 64 * r;
+            S[c][r] = (d < D && c0 + c < V) ? Sg[(size_t)d * V + c0 + c] : 0.0f;
+        }
+    float q[RPL], k[RPL], g[RPL], vv[kDeltaCols], bt;
+    auto fetch = [&](int t, float* fq, float* fk, float* fg, float* fv, float& fb) {
         const size_t m = (size_t)(m0 + t);
 #pragma unroll
-        for (int i = 0; i < kPre; ++i) {
-            const int idx = tid + 256 * i;
-            float val = 0.0f;
-            if (idx < D) val = qk[m * ldqk + (size_t)kvh * D + idx];
-            else if (idx < 2 * D) val = qk[m * ldqk + (size_t)(G + kvh) * D + (idx - D)];
-            else if (idx < 3 * D) val = dec[m * ldd + (size_t)h * D + (idx - 2 * D)];
-            else if (idx < 3 * D + V) val = v[m * ldv + (size_t)h * V + (idx - 3 * D)];
-            else if (idx == 3 * D + V) val = beta[m * ldb + h];
-            pre[i] = val;
+        for (int r = 0; r < RPL; ++r) {
+            const int d = lane + 64 * r;
+            const bool ok = d < D;
+            fq[r] = ok ? qk[m * ldqk + (size_t)kvh * D + d] : 0.0f;
+            fk[r] = ok ? qk[m * ldqk + (size_t)(G + kvh) * D + d] : 0.0f;
+            fg[r] = ok ? dec[m * ldd + (size_t)h * D + d] : 0.0f;
         }
-    };
-    auto stash = [&](int buf, const float pre[kPre]) {
 #pragma unroll
-        for (int i = 0; i < kPre; ++i) {
-            const int idx = tid + 256 * i;
-            if (idx < n_stage) s_stage[buf * n_stage + idx] = pre[i];
-        }
+        for (int c = 0; c < kDeltaCols; ++c) fv[c] = c0 + c < V ? v[m * ldv + (size_t)h * V + c0 + c] : 0.0f;
+        fb = beta[m * ldb + h];
     };
-    float pre[kPre];
-    fetch(0, pre);
-    stash(0, pre);
+    fetch(0, q, k, g, vv, bt);
     for (int t = 0; t < n; ++t) {
-        if (t + 1 < n) fetch(t + 1, pre);
-        __syncthreads();  // the token's vectors are staged
-        const float* sq = s_stage + (t & 1) * n_stage;
-        const float *sk = sq + D, *sg = sk + D, *sv = sg + D;
-        const float bt = sv[V];
-        float part = 0.0f;
+        float nq[RPL], nk[RPL], ng[RPL], nv[kDeltaCols], nb = 0.0f;
+        if (t + 1 < n) fetch(t + 1, nq, nk, ng, nv, nb);
+        float part[kDeltaCols];
 #pragma unroll
-        for (int r = 0; r < RPT; ++r) {
-            const int d = rg + NR * r;
-            if (d < D) {
-                S[r] *= sg[d];
-                part = fmaf(S[r], sk[d], part);
-            }
-        }
-        s_p1[rg * VP + c] = part;
-        __syncthreads();
-        float kv = 0.0f;
-        for (int g2 = 0; g2 < NR; ++g2) kv += s_p1[g2 * VP + c];
-        const float u = col_ok ? bt * (sv[c] - kv) : 0.0f;
-        float part2 = 0.0f;
+        for (int c = 0; c < kDeltaCols; ++c) {
+            float a = 0.0f;
 #pragma unroll
-        for (int r = 0; r < RPT; ++r) {
-            const int d = rg + NR * r;
-            if (d < D) {
-                S[r] = fmaf(sk[d], u, S[r]);
-                part2 = fmaf(S[r], sq[d], part2);
+            for (int r = 0; r < RPL; ++r) {
+                S[c][r] *= g[r];
+                a = fmaf(S[c][r], k[r], a);
             }
+            part[c] = a;
         }
-        s_p2[rg * VP + c] = part2;
-        if (t + 1 < n) stash((t + 1) & 1, pre);
-        __syncthreads();
-        if (rg == 0 && col_ok) {
-            float o = 0.0f;
-            for (int g2 = 0; g2 < NR; ++g2) o += s_p2[g2 * VP + c];
-            out[(size_t)(m0 + t) * ldo + (size_t)h * V + c] = o;
+#pragma unroll
+        for (int c = 0; c < kDeltaCols; ++c) part[c] = wave_allsum(part[c]);
+#pragma unroll
+        for (int c = 0; c < kDeltaCols; ++c) {
+            const float u = bt * (vv[c] - part[c]);
+            float a = 0.0f;
+#pragma unroll
+            for (int r = 0; r < RPL; ++r) {
+                S[c][r] = fmaf(k[r], u, S[c][r]);
+                a = fmaf(S[c][r], q[r], a);
+            }
+            part[c] = a;
+        }
+#pragma unroll
+        for (int c = 0; c < kDeltaCols; ++c) part[c] = wave_allsum(part[c]);
+        if (lane < kDeltaCols && c0 + lane < V) {
+            float o = part[0];
+#pragma unroll
+            for (int c = 1; c < kDeltaCols; ++c) o = lane == c ? part[c] : o;
+            out[(size_t)(m0 + t) * ldo + (size_t)h * V + c0 + lane] = o;
+        }
+        if (t + 1 < n) {
+#pragma unroll
+            for (int r = 0; r < RPL; ++r) {
+                q[r] = nq[r];
+                k[r] = nk[r];
+                g[r] = ng[r];
+            }
+#pragma unroll
+            for (int c = 0; c < kDeltaCols; ++c) vv[c] = nv[c];
+            bt = nb;
         }
     }
 #pragma unroll
-    for (int r = 0; r < RPT; ++r) {
-        const int d = rg + NR * r;
-        if (col_ok && d < D) Sg[(size_t)d * V + c] = S[r];
-    }
+    for (int c = 0; c < kDeltaCols; ++c)
+#pragma unroll
+        for (int r = 0; r < RPL; ++r) {
+            const int d = lane + 64 * r;
+            if (d < D && c0 + c < V) Sg[(size_t)d * V + c0 + c] = S[c][r];
+        }
 }
 
 // one wave per (row, head) vector, in place: v / rms(v) * w * sigmoid(gate)
@@ -489,11 +683,54 @@ int launch_window_attention(const float* q, int ldq, float* out, int ldo, int M,
     return ZG_OK;
 }
 
+size_t window_split_workspace(int rows, int H, int V, int key_capacity, int* n_split_out) {
+    const int n_split = std::max(1, std::min(kWinSplits, (key_capacity + kMixTile - 1) / kMixTile));
+    if (n_split_out) *n_split_out = n_split;
+    return (size_t)rows * H * key_capacity + (size_t)rows * n_split * H * 2 + (size_t)rows * n_split * H * V;
+}
+
+int launch_window_attention_split(const float* q, int ldq, float* out, int ldo, int M, int H, int G, int D, int V, float scale, int window,
+                                  const float* sink, const float* talk, const float* vfreq, const int* row_pos, const int* row_slot,
+                                  const int* page_table, int max_pages, int page_tokens, const float* cache, int key_capacity, float* ws,
+                                  size_t ws_floats, hipStream_t s, bool* taken) {
+    *taken = false;
+    if (M <= 0) return ZG_OK;
+    if (const char* e = getenv("ZGPT2_LM_WINDOW_GENERAL"))  // test hook: every step through the general kernel
+        if (atoi(e) != 0) return ZG_OK;
+    int n_split = 1;
+    const size_t need = window_split_workspace(M, H, V, key_capacity, &n_split);
+    const int rpl = (D + 63) / 64;
+    const size_t lds_a = ((size_t)H * 64 * rpl + 8 * (size_t)H) * sizeof(float);
+    const size_t lds_b = (2 * (size_t)H * kMixTile + (size_t)H * H + 2 * (size_t)H) * sizeof(float);
+    if (!ws || need > ws_floats || H > kWinMaxHeads || H % G != 0 || H * V > 256 * kWinAcc || D > 256 || V % 2 != 0 || lds_a > 60 * 1024 ||
+        lds_b > 60 * 1024 || M > 65535)
+        return ZG_OK;  // the general kernel takes it
+    float* sc = ws;
+    float* st = sc + (size_t)M * H * key_capacity;
+    float* po = st + (size_t)M * n_split * H * 2;
+    const dim3 grid(n_split, M);
+#define ZG_WS(R)                                                                                                                              \
+    window_scores_kernel<R><<<grid, 256, lds_a, s>>>(q, ldq, H, G, D, V, scale, window, row_pos, row_slot, page_table, max_pages, page_tokens, cache, \
+                                                     sc, key_capacity, st)
+    if (rpl <= 1) ZG_WS(1);
+    else if (rpl <= 2) ZG_WS(2);
+    else ZG_WS(4);
+#undef ZG_WS
+    ZG_HIP(hipGetLastError());
+    window_mix_kernel<<<grid, 256, lds_b, s>>>(H, G, D, V, window, sink, talk, row_pos, row_slot, page_table, max_pages, page_tokens, cache, sc,
+                                               key_capacity, st, po);
+    ZG_HIP(hipGetLastError());
+    window_merge_kernel<<<M, 256, 0, s>>>(po, n_split, out, ldo, H, V, vfreq, row_pos);
+    ZG_HIP(hipGetLastError());
+    *taken = true;
+    return ZG_OK;
+}
+
 int launch_rglru_scan(const float* u, int ldu, const float* gr, const float* gi, int ldg, const float* br, const float* bi, const float* lam,
                       const float* y, int ldy, const float* by, float* out, int ldo, int C, float* state, size_t slot_stride, const int* ent_start,
                       const int* ent_len, const int* ent_slot, int n_entries, hipStream_t s) {
     if (n_entries <= 0 || C <= 0) return ZG_OK;
-    rglru_scan_kernel<<<dim3(n_entries, (C + 63) / 64), 64, 0, s>>>(u, ldu, gr, gi, ldg, br, bi, lam, y, ldy, by, out, ldo, C, state, slot_stride,
+    rglru_scan_kernel<<<dim3(n_entries, (C + 63) / 64), 64 * kLruSegs, 0, s>>>(u, ldu, gr, gi, ldg, br, bi, lam, y, ldy, by, out, ldo, C, state, slot_stride,
                                                                   ent_start, ent_len, ent_slot);
     ZG_HIP(hipGetLastError());
     return ZG_OK;
@@ -520,20 +757,13 @@ int launch_delta_scan(const float* qk, int ldqk, const float* v, int ldv, const 
     if (n_entries <= 0) return ZG_OK;
     ZG_REQUIRE(D >= 1 && D <= 256 && V >= 1 && V <= 256 && G >= 1 && H % G == 0, ZG_ERR_UNSUPPORTED,
                "delta rule: %d heads on %d key heads, %d key and %d value channels per head (at most 256 each)", H, G, D, V);
-    int VP = 1;
-    while (VP < V) VP <<= 1;
-    const int NR = 256 / VP, rpt = (D + NR - 1) / NR;
-    ZG_REQUIRE(rpt <= 64, ZG_ERR_UNSUPPORTED, "delta rule: a state of %d x %d per head (at most 16384 elements)", D, V);
-    const size_t lds = (2 * (size_t)(3 * D + V + 1) + 2 * 256) * sizeof(float);
-    const dim3 grid(n_entries, H);
-#define ZG_DELTA(R)                                                                                                                          \
-    delta_scan_kernel<R><<<grid, 256, lds, s>>>(qk, ldqk, v, ldv, beta, ldb, dec, ldd, out, ldo, H, G, D, V, VP, state, slot_stride, ent_start, \
-                                                ent_len, ent_slot)
-    if (rpt <= 4) ZG_DELTA(4);
-    else if (rpt <= 8) ZG_DELTA(8);
-    else if (rpt <= 16) ZG_DELTA(16);
-    else if (rpt <= 32) ZG_DELTA(32);
-    else ZG_DELTA(64);
+    const int rpl = (D + 63) / 64;
+    const dim3 grid(n_entries, H, (V + 4 * kDeltaCols - 1) / (4 * kDeltaCols));
+#define ZG_DELTA(R) \
+    delta_scan_kernel<R><<<grid, 256, 0, s>>>(qk, ldqk, v, ldv, beta, ldb, dec, ldd, out, ldo, H, G, D, V, state, slot_stride, ent_start, ent_len, ent_slot)
+    if (rpl <= 1) ZG_DELTA(1);
+    else if (rpl <= 2) ZG_DELTA(2);
+    else ZG_DELTA(4);
 #undef ZG_DELTA
     ZG_HIP(hipGetLastError());
     return ZG_OK;
