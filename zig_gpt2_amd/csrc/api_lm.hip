@@ -242,7 +242,7 @@ void layout(zg_lm* g, Bump& b) {
         mat("head", g->head, 0, V, W);
     }
     vec("final.norm", g->final_norm, W, INIT_OFFSET);
-    size_t max_t = 1, max_win = 0;
+    size_t max_t = 1, max_win = 0, max_win_few = 0;
     size_t max_proj = 1, max_qr = 1, max_q = 1, max_qa = 1, max_ctx = 1, max_o = 1, max_ff = 1, max_assign = 1, max_gu = 1, max_hb = 1, max_e = 1, max_att_part = 0, max_scan = 0;
     for (size_t i = 0; i < g->layers.size(); ++i) {
         LayerW& L = g->layers[i];
@@ -287,7 +287,9 @@ void layout(zg_lm* g, Bump& b) {
             max_proj = std::max(max_proj, NP);
             max_o = std::max(max_o, HV);
             max_t = std::max(max_t, C);
-            max_win = std::max(max_win, window_split_workspace((int)MS, (int)H, (int)Vd, d.window > 0 ? d.window : g->max_pages * g->P, nullptr));
+            const int cap = d.window > 0 ? d.window : g->max_pages * g->P;
+            max_win = std::max(max_win, window_split_workspace((int)MS, (int)H, (int)Vd, cap, nullptr));
+            max_win_few = std::max(max_win_few, window_split_workspace(kGemvMaxRows, (int)H, (int)Vd, cap, nullptr));
         } else if (d.mixer == ZG_LM_MIX_CHANNEL_DELTA) {
             const size_t G = d.kv_heads, HV = H * Vd, CC = 2 * G * D + HV, RA = d.decay_rank, RG = d.gate_rank;
             const size_t NP = CC + H + RA + RG;
@@ -458,7 +460,8 @@ void layout(zg_lm* g, Bump& b) {
     g->attn_ws = b.take<float>(std::max<size_t>(1, g->attn_ws_floats));
     // scores and partial sums of the split windowed attention: up to 2 GiB for a whole portion, else for steps of few rows only
     // (longer steps of such a model then take the general kernel)
-    if (max_win > ((size_t)1 << 29)) max_win = max_win / MS * kGemvMaxRows;
+    if (max_win > ((size_t)1 << 29)) max_win = 0;
+    max_win = std::max(max_win, max_win_few);
     if (max_win > ((size_t)1 << 29)) max_win = 0;
     g->win_ws_floats = max_win;
     g->win_ws = b.take<float>(std::max<size_t>(1, max_win));
@@ -575,7 +578,7 @@ int enqueue_layers(zg_lm* g, int M, int n_ent, bool capturing, bool single) {
         ConvArgs c;
         c.in = g->h; c.ld_in = W; c.out = g->hc; c.ld_out = W; c.C = W; c.taps = g->canon; c.w = w; c.flags = CONV_RESIDUAL;
         c.tail = g->seq_state + off; c.slot_stride = g->seq_floats;
-        return launch_causal_conv(c, M, n_ent, d_off, d_slot, d_estart, d_elen, d_eslot, s);
+        return launch_causal_conv(c, M, n_ent, single, d_off, d_slot, d_estart, d_elen, d_eslot, s);
     };
     bool h_ready = false;  // g->h already holds this pass's shifted norm (written by the previous pass's fused tail)
     for (int p = 0; p < g->n_passes; ++p) {
@@ -583,14 +586,18 @@ int enqueue_layers(zg_lm* g, int M, int n_ent, bool capturing, bool single) {
         const LayerW& L = g->layers[ps.layer];
         const zg_lm_layer& d = L.d;
         const int H = d.heads, D = d.dim, Vd = d.vdim;
-        if (ps.readd) ZG_TRY(launch_add_rows(g->x, g->x0, M, W, s));
-        if (!h_ready)
+        bool hc_ready = false;  // one launch has done everything up to the mixer's input (decode steps)
+        if (canon && single && !h_ready)
+            ZG_TRY(launch_norm_conv_single(g->x, ps.readd ? g->x0 : nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, L.norm1, eps, M, W, g->canon,
+                                           L.canon1, g->seq_state + ps.canon1_off, g->seq_floats, d_slot, g->hc, s, &hc_ready));
+        if (ps.readd && !hc_ready) ZG_TRY(launch_add_rows(g->x, g->x0, M, W, s));
+        if (!h_ready && !hc_ready)
             ZG_TRY(launch_norm_shift(g->x, L.norm1, canon ? nullptr : L.shift, eps, g->h, M, W, d_prev, d_slot, g->shift_state + (size_t)p * W,
                                      (size_t)g->n_passes * W, canon ? nullptr : d_last, g->last_h + (size_t)p * NS * W, s));
         h_ready = false;
         const float* hin = g->h;  // what the sublayer reads
         if (canon) {
-            ZG_TRY(input_conv(L.canon1, ps.canon1_off));
+            if (!hc_ready) ZG_TRY(input_conv(L.canon1, ps.canon1_off));
             hin = g->hc;
         }
         // one row per entry: the pass's last sum is fused with the next pass's norm + shift (tail below)
@@ -601,6 +608,7 @@ int enqueue_layers(zg_lm* g, int M, int n_ent, bool capturing, bool single) {
                                          (size_t)g->n_passes * W, d_last, g->last_h + (size_t)(p + 1) * NS * W, s, &h_ready);
         };
         Linear lin;
+        bool mid_done = false;  // x, and the feed-forward's input in g->hc, are already there
         if (d.mixer == ZG_LM_MIX_PARALLEL) {
             const int G = d.kv_heads, C = d.lru_width, NB = d.lru_blocks, BS = C / NB, HV = H * Vd, NP = L.n_cat;
             const int oy = H * D + G * D + G * Vd, ox = oy + C;  // columns of the two branches of the recurrent unit
@@ -624,7 +632,7 @@ int enqueue_layers(zg_lm* g, int M, int n_ent, bool capturing, bool single) {
             ConvArgs cv;
             cv.in = g->proj + ox; cv.ld_in = NP; cv.out = g->ta; cv.ld_out = C; cv.C = C; cv.taps = d.lru_conv; cv.w = L.convw; cv.bias = L.convb;
             cv.pre_bias = L.xb; cv.tail = g->seq_state + ps.conv_off; cv.slot_stride = g->seq_floats;
-            ZG_TRY(launch_causal_conv(cv, M, n_ent, d_off, d_slot, d_estart, d_elen, d_eslot, s));
+            ZG_TRY(launch_causal_conv(cv, M, n_ent, single, d_off, d_slot, d_estart, d_elen, d_eslot, s));
             for (int which = 0; which < 2; ++which) {
                 lin = Linear();
                 lin.A = g->ta; lin.lda = C; lin.a_zoff = BS; lin.B = which ? L.ri : L.ra; lin.ldb = BS; lin.b_zoff = (long long)BS * BS;
@@ -636,7 +644,10 @@ int enqueue_layers(zg_lm* g, int M, int n_ent, bool capturing, bool single) {
             lin = Linear();
             lin.A = g->td; lin.lda = C; lin.B = L.ro; lin.ldb = C; lin.C = g->y2; lin.ldc = W; lin.M = M; lin.N = W; lin.K = C;
             ZG_TRY(launch_linear(lin, f32, s));
-            ZG_TRY(launch_pair_norm_mean(g->y, g->y2, L.left_out, L.right_out, eps, g->y, M, W, s));
+            if (canon && single && d.ff != ZG_LM_FF_NONE)  // the branches' mean, the residual sum, the next norm and its convolution at once
+                ZG_TRY(launch_norm_conv_single(g->x, nullptr, g->y, g->y2, L.left_out, L.right_out, L.norm1b, L.norm2, eps, M, W, g->canon, L.canon2,
+                                               g->seq_state + ps.canon2_off, g->seq_floats, d_slot, g->hc, s, &mid_done));
+            if (!mid_done) ZG_TRY(launch_pair_norm_mean(g->y, g->y2, L.left_out, L.right_out, eps, g->y, M, W, s));
         } else if (d.mixer == ZG_LM_MIX_CHANNEL_DELTA) {
             const int G = d.kv_heads, HV = H * Vd, CC = 2 * G * D + HV, RA = d.decay_rank, RG = d.gate_rank, NP = L.n_cat;
             lin = Linear();
@@ -645,7 +656,7 @@ int enqueue_layers(zg_lm* g, int M, int n_ent, bool capturing, bool single) {
             ConvArgs cv;
             cv.in = g->proj; cv.ld_in = NP; cv.out = g->ta; cv.ld_out = CC; cv.C = CC; cv.taps = d.conv; cv.w = L.convw; cv.flags = CONV_SILU;
             cv.tail = g->seq_state + ps.conv_off; cv.slot_stride = g->seq_floats;
-            ZG_TRY(launch_causal_conv(cv, M, n_ent, d_off, d_slot, d_estart, d_elen, d_eslot, s));
+            ZG_TRY(launch_causal_conv(cv, M, n_ent, single, d_off, d_slot, d_estart, d_elen, d_eslot, s));
             lin = Linear();  // the decay's second step
             lin.A = g->proj + CC + H; lin.lda = NP; lin.B = L.a2; lin.ldb = RA; lin.C = g->tb; lin.ldc = H * D; lin.M = M; lin.N = H * D; lin.K = RA;
             ZG_TRY(launch_linear(lin, f32, s));
@@ -701,7 +712,11 @@ int enqueue_layers(zg_lm* g, int M, int n_ent, bool capturing, bool single) {
             lin.A = g->o; lin.lda = HV; lin.B = L.o; lin.ldb = HV; lin.C = g->y; lin.ldc = W; lin.M = M; lin.N = W; lin.K = HV;
             ZG_TRY(launch_linear(lin, f32, s));
         }
-        if (d.ff != ZG_LM_FF_NONE) ZG_TRY(launch_norm_add_norm(g->x, g->y, L.norm1b, L.norm2, eps, g->h, M, W, s));
+        if (canon && single && d.ff != ZG_LM_FF_NONE && !mid_done)
+            ZG_TRY(launch_norm_conv_single(g->x, nullptr, g->y, nullptr, nullptr, nullptr, L.norm1b, L.norm2, eps, M, W, g->canon, L.canon2,
+                                           g->seq_state + ps.canon2_off, g->seq_floats, d_slot, g->hc, s, &mid_done));
+        if (mid_done) {
+        } else if (d.ff != ZG_LM_FF_NONE) ZG_TRY(launch_norm_add_norm(g->x, g->y, L.norm1b, L.norm2, eps, g->h, M, W, s));
         else {
             ZG_TRY(tail(g->y, nullptr, nullptr, 0, L.norm1b));
             if (!h_ready) ZG_TRY(launch_norm_add(g->x, g->y, L.norm1b, eps, M, W, s));
@@ -709,7 +724,7 @@ int enqueue_layers(zg_lm* g, int M, int n_ent, bool capturing, bool single) {
         const int F = d.ff_width;
         hin = g->h;
         if (canon && d.ff != ZG_LM_FF_NONE) {
-            ZG_TRY(input_conv(L.canon2, ps.canon2_off));
+            if (!mid_done) ZG_TRY(input_conv(L.canon2, ps.canon2_off));
             hin = g->hc;
         }
         if (d.ff == ZG_LM_FF_DENSE) {

@@ -131,8 +131,15 @@ struct ConvArgs {
     float* tail = nullptr;
     size_t slot_stride = 0;
 };
-int launch_causal_conv(const ConvArgs& a, int M, int n_entries, const int* row_off, const int* row_slot, const int* ent_start, const int* ent_len,
-                       const int* ent_slot, hipStream_t s);
+// one_row_each: every entry brings exactly one row (decode steps): the convolution's own threads move the tails on, no second launch.
+int launch_causal_conv(const ConvArgs& a, int M, int n_entries, bool one_row_each, const int* row_off, const int* row_slot, const int* ent_start,
+                       const int* ent_len, const int* ent_slot, hipStream_t s);
+// Steps of one row per entry: [x += x0] or [x += norm(y) * (1 + wb), y = yl or the mean of the two normed branches yl, yr with
+// plain weights wl, wr], then h = norm(x) * (1 + wn), out = h + conv(h) over the slot's tail, the tail moved on — one launch.
+// *taken = false for rows too wide for its registers (nothing launched).
+int launch_norm_conv_single(float* x, const float* x0, const float* yl, const float* yr, const float* wl, const float* wr, const float* wb,
+                            const float* wn, float eps, int M, int W, int taps, const float* cw, float* tail, size_t slot_stride,
+                            const int* row_slot, float* out, hipStream_t s, bool* taken);
 // x[m] += y[m]
 int launch_add_rows(float* x, const float* y, int M, int W, hipStream_t s);
 
@@ -153,7 +160,7 @@ int launch_window_attention(const float* q, int ldq, float* out, int ldo, int M,
 // steps of few rows need to fill the chip, and prompt portions to compute every score once.  key_capacity: the most keys a row
 // can see (the window, or the longest sequence).  ws: window_split_workspace(rows, ...) floats.  *taken = false (nothing
 // launched) when the workspace is too small or a size is beyond the kernels' limits.
-constexpr int kWinSplits = 16;
+constexpr int kWinSplits = 64;
 size_t window_split_workspace(int rows, int H, int V, int key_capacity, int* n_split_out);
 int launch_window_attention_split(const float* q, int ldq, float* out, int ldo, int M, int H, int G, int D, int V, float scale, int window,
                                   const float* sink, const float* talk, const float* vfreq, const int* row_pos, const int* row_slot,

@@ -43,30 +43,38 @@ __global__ __launch_bounds__(256) void add_rows_kernel(float* x, const float* y,
 // ------------------------------------------------------------------------------------------------ causal convolution
 // Tap j of row m reads the input taps - 1 - j tokens back: a row of the same step when the entry brought that many tokens in
 // front of m, else the slot's tail (the taps - 1 inputs before the step, oldest first; zeros for a new sequence).
+constexpr int kMaxTaps = 16;
 __global__ __launch_bounds__(256) void causal_conv_kernel(const float* in, int ld_in, float* out, int ld_out, int C, int taps, const float* w,
-                                                          const float* bias, const float* pre_bias, int flags, const float* tail,
-                                                          size_t slot_stride, const int* row_off, const int* row_slot) {
+                                                          const float* bias, const float* pre_bias, int flags, float* tail, size_t slot_stride,
+                                                          const int* row_off, const int* row_slot, int own_tail) {
     const int m = blockIdx.x, c = blockIdx.y * blockDim.x + threadIdx.x;
     if (c >= C) return;
     const int off = row_off[m], K = taps - 1;
-    const float* tl = tail + (size_t)row_slot[m] * slot_stride;
+    float* tl = tail + (size_t)row_slot[m] * slot_stride;
     const float pb = pre_bias ? pre_bias[c] : 0.0f;  // a bias of the input itself (the tail holds inputs with it)
     float acc = bias ? bias[c] : 0.0f;
-    float cur = 0.0f;
-    for (int j = 0; j < taps; ++j) {
-        const int src = off - K + j;
-        const float v = src >= 0 ? in[(size_t)(m - K + j) * ld_in + c] + pb : tl[(size_t)(K + src) * C + c];
-        acc = fmaf(w[(size_t)c * taps + j], v, acc);
-        cur = v;
+    float val[kMaxTaps];
+#pragma unroll
+    for (int j = 0; j < kMaxTaps; ++j) {
+        val[j] = 0.0f;
+        if (j < taps) {
+            const int src = off - K + j;
+            val[j] = src >= 0 ? in[(size_t)(m - K + j) * ld_in + c] + pb : tl[(size_t)(K + src) * C + c];
+            acc = fmaf(w[(size_t)c * taps + j], val[j], acc);
+        }
     }
-    if (flags & CONV_RESIDUAL) acc += cur;
+    if (flags & CONV_RESIDUAL) acc += in[(size_t)m * ld_in + c] + pb;
     if (flags & CONV_SILU) acc = silu_f(acc);
     out[(size_t)m * ld_out + c] = acc;
+    if (own_tail) {  // the row is its entry's only one: this thread has read its channel's whole tail and moves it on itself
+#pragma unroll
+        for (int i = 0; i + 1 < kMaxTaps; ++i)
+            if (i < K) tl[(size_t)i * C + c] = val[i + 1];
+    }
 }
 
 // The new tail of every entry's slot: the last taps - 1 of (old tail, the entry's inputs).  A thread reads all it needs
 // before it writes, and no other thread touches its channel of its slot.
-constexpr int kMaxTaps = 16;
 __global__ __launch_bounds__(256) void conv_tail_kernel(const float* in, int ld_in, int C, int taps, const float* pre_bias, float* tail,
                                                         size_t slot_stride, const int* ent_start, const int* ent_len, const int* ent_slot) {
     const int e = blockIdx.x, c = blockIdx.y * blockDim.x + threadIdx.x;
@@ -85,6 +93,79 @@ __global__ __launch_bounds__(256) void conv_tail_kernel(const float* in, int ld_
 #pragma unroll
     for (int i = 0; i < kMaxTaps; ++i)
         if (i < K) tl[(size_t)i * C + c] = val[i];
+}
+
+// Decode steps (one row per entry), rows of up to 256 * kSingleRegs floats held in registers: everything between two matrix
+// products of a layer pass in one launch —
+//   [x += x0]   or   [y = yl, or the mean of the two normed branches (yl / rms * wl + yr / rms * wr) / 2;  x += y / rms(y) * (1 + wb)]
+//   h = x / rms(x) * (1 + wn);   out = h + conv(h) over the slot's tail;   the tail moved on by h.
+constexpr int kSingleRegs = 16;
+__global__ __launch_bounds__(256) void norm_conv_single_kernel(float* x, const float* x0, const float* yl, const float* yr, const float* wl,
+                                                               const float* wr, const float* wb, const float* wn, float eps, int W, int taps,
+                                                               const float* cw, float* tail, size_t slot_stride, const int* row_slot,
+                                                               float* out) {
+    __shared__ float s_red[8];
+    const int m = blockIdx.x, K = taps - 1;
+    float* xr = x + (size_t)m * W;
+    float* tl = tail + (size_t)row_slot[m] * slot_stride;
+    float xv[kSingleRegs], yv[kSingleRegs];
+#pragma unroll
+    for (int j = 0; j < kSingleRegs; ++j) {
+        const int i = threadIdx.x + 256 * j;
+        xv[j] = i < W ? xr[i] + (x0 ? x0[(size_t)m * W + i] : 0.0f) : 0.0f;
+        yv[j] = (i < W && yl) ? yl[(size_t)m * W + i] : 0.0f;
+    }
+    if (yl) {
+        if (yr) {
+            float zv[kSingleRegs], sa = 0.0f, sb = 0.0f;
+#pragma unroll
+            for (int j = 0; j < kSingleRegs; ++j) {
+                const int i = threadIdx.x + 256 * j;
+                zv[j] = i < W ? yr[(size_t)m * W + i] : 0.0f;
+                sa = fmaf(yv[j], yv[j], sa);
+                sb = fmaf(zv[j], zv[j], sb);
+            }
+            sa = block_allsum(sa, s_red);
+            sb = block_allsum(sb, s_red);
+            const float ra = 1.0f / sqrtf(sa / (float)W + eps), rb = 1.0f / sqrtf(sb / (float)W + eps);
+#pragma unroll
+            for (int j = 0; j < kSingleRegs; ++j) {
+                const int i = threadIdx.x + 256 * j;
+                yv[j] = i < W ? 0.5f * (yv[j] * ra * wl[i] + zv[j] * rb * wr[i]) : 0.0f;
+            }
+        }
+        float sy = 0.0f;
+#pragma unroll
+        for (int j = 0; j < kSingleRegs; ++j) sy = fmaf(yv[j], yv[j], sy);
+        sy = block_allsum(sy, s_red);
+        const float ry = 1.0f / sqrtf(sy / (float)W + eps);
+#pragma unroll
+        for (int j = 0; j < kSingleRegs; ++j) {
+            const int i = threadIdx.x + 256 * j;
+            if (i < W) xv[j] += yv[j] * ry * (1.0f + wb[i]);
+        }
+    }
+    float sx = 0.0f;
+#pragma unroll
+    for (int j = 0; j < kSingleRegs; ++j) sx = fmaf(xv[j], xv[j], sx);
+    sx = block_allsum(sx, s_red);
+    const float rx = 1.0f / sqrtf(sx / (float)W + eps);
+#pragma unroll
+    for (int j = 0; j < kSingleRegs; ++j) {
+        const int i = threadIdx.x + 256 * j;
+        if (i < W) {
+            if (x0 || yl) xr[i] = xv[j];
+            const float h = xv[j] * rx * (1.0f + wn[i]);
+            float acc = cw[(size_t)i * taps + K] * h;
+            for (int t = 0; t < K; ++t) {  // tail entry t is taps - 1 - t tokens back; it moves one place towards the front
+                const float tv = tl[(size_t)t * W + i];
+                acc = fmaf(cw[(size_t)i * taps + t], tv, acc);
+                if (t > 0) tl[(size_t)(t - 1) * W + i] = tv;
+            }
+            if (K > 0) tl[(size_t)(K - 1) * W + i] = h;
+            out[(size_t)m * W + i] = h + acc;
+        }
+    }
 }
 
 // ------------------------------------------------------------------------------------------------ windowed attention
@@ -267,14 +348,19 @@ __device__ __forceinline__ void window_range(int pos, int window, int n_split, i
     k1 = min(n_keys, k0 + chunk);
 }
 
+constexpr int kScoreTile = 128;  // keys whose scores a workgroup holds in the LDS at a time
+constexpr int kScoreKeys = 4;    // keys a wave has in flight
+
 template <int RPL>
 __global__ __launch_bounds__(256) void window_scores_kernel(const float* q, int ldq, int H, int G, int D, int V, float scale, int window,
                                                             const int* row_pos, const int* row_slot, const int* page_table, int max_pages,
                                                             int page_tokens, const float* cache, float* sc, int NK, float* st) {
     extern __shared__ __attribute__((aligned(16))) float s_sc[];
-    float* s_q = s_sc;           // [H][64 RPL] (zero beyond D)
-    float* s_m = s_q + H * 64 * RPL;  // [4][H]
-    float* s_l = s_m + 4 * H;         // [4][H]
+    float* s_q = s_sc;                     // [H][64 RPL] (zero beyond D)
+    float* s_t = s_q + H * 64 * RPL;       // [H][kScoreTile] scores of the tile
+    float* s_m = s_t + H * kScoreTile;     // [H] running maximum
+    float* s_l = s_m + H;                  // [H] running sum of exp
+    __shared__ int s_row[kScoreTile];
     const int split = blockIdx.x, n_split = gridDim.x, m = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int pos = row_pos[m];
     int j_lo, k0, k1;
@@ -286,43 +372,69 @@ __global__ __launch_bounds__(256) void window_scores_kernel(const float* q, int 
         const int h = i / (64 * RPL), d = i % (64 * RPL);
         s_q[i] = d < D ? q[(size_t)m * ldq + (size_t)h * D + d] : 0.0f;
     }
-    for (int i = threadIdx.x; i < 4 * H; i += blockDim.x) {
+    for (int i = threadIdx.x; i < H; i += blockDim.x) {
         s_m[i] = -INFINITY;
         s_l[i] = 0.0f;
     }
-    __syncthreads();
     float* srow = sc + (size_t)m * H * NK;
-    for (int kk = k0 + wave; kk < k1; kk += 4) {
-        const int j = j_lo + kk;
-        const float* kr = cache + ((size_t)pages[(j / page_tokens) % max_pages] * page_tokens + j % page_tokens) * cstride;
-        for (int g = 0; g < G; ++g) {
-            float kd[RPL];
+    for (int t0 = k0; t0 < k1; t0 += kScoreTile) {
+        const int nt = min(kScoreTile, k1 - t0);
+        __syncthreads();  // the tile before has been consumed (and, the first time, q is staged)
+        for (int i = threadIdx.x; i < nt; i += blockDim.x) {
+            const int j = j_lo + t0 + i;
+            s_row[i] = pages[(j / page_tokens) % max_pages] * page_tokens + j % page_tokens;
+        }
+        __syncthreads();
+        // a wave takes kScoreKeys keys at a time: all their loads are requested before the first product
+        for (int kk = wave * kScoreKeys; kk < nt; kk += 4 * kScoreKeys) {
+            for (int g = 0; g < G; ++g) {
+                float kd[kScoreKeys][RPL];
 #pragma unroll
-            for (int r = 0; r < RPL; ++r) kd[r] = lane + 64 * r < D ? kr[(size_t)g * D + lane + 64 * r] : 0.0f;
-            for (int hh = 0; hh < rep; ++hh) {
-                const int h = g * rep + hh;
-                float a = 0.0f;
+                for (int u = 0; u < kScoreKeys; ++u) {
+                    const float* kr = cache + (size_t)s_row[min(kk + u, nt - 1)] * cstride + (size_t)g * D;
 #pragma unroll
-                for (int r = 0; r < RPL; ++r) a = fmaf(s_q[h * 64 * RPL + lane + 64 * r], kd[r], a);
-                a = wave_allsum(a) * scale;
-                if (lane == 0) {
-                    srow[(size_t)h * NK + kk] = a;
-                    const float mo = s_m[wave * H + h], mn = fmaxf(mo, a);
-                    s_l[wave * H + h] = s_l[wave * H + h] * expf(mo - mn) + expf(a - mn);
-                    s_m[wave * H + h] = mn;
+                    for (int r = 0; r < RPL; ++r) kd[u][r] = lane + 64 * r < D ? kr[lane + 64 * r] : 0.0f;
                 }
+                for (int hh = 0; hh < rep; ++hh) {
+                    const int h = g * rep + hh;
+                    float a[kScoreKeys];
+#pragma unroll
+                    for (int u = 0; u < kScoreKeys; ++u) {
+                        a[u] = 0.0f;
+#pragma unroll
+                        for (int r = 0; r < RPL; ++r) a[u] = fmaf(s_q[h * 64 * RPL + lane + 64 * r], kd[u][r], a[u]);
+                    }
+#pragma unroll
+                    for (int u = 0; u < kScoreKeys; ++u) a[u] = wave_allsum(a[u]) * scale;
+                    if (lane < kScoreKeys && kk + lane < nt) {
+                        float mine = a[0];
+#pragma unroll
+                        for (int u = 1; u < kScoreKeys; ++u) mine = lane == u ? a[u] : mine;
+                        s_t[h * kScoreTile + kk + lane] = mine;
+                        srow[(size_t)h * NK + t0 + kk + lane] = mine;
+                    }
+                }
+            }
+        }
+        __syncthreads();
+        for (int h = wave; h < H; h += 4) {  // the tile's share of the head's maximum and sum, a wave per head
+            float mx = -INFINITY;
+            for (int i = lane; i < nt; i += 64) mx = fmaxf(mx, s_t[h * kScoreTile + i]);
+            mx = fmaxf(wave_allmax(mx), s_m[h]);
+            float l = 0.0f;
+            for (int i = lane; i < nt; i += 64) l += expf(s_t[h * kScoreTile + i] - mx);
+            l = wave_allsum(l);
+            if (lane == 0) {
+                s_l[h] = (s_l[h] > 0.0f ? s_l[h] * expf(s_m[h] - mx) : 0.0f) + l;
+                s_m[h] = mx;
             }
         }
     }
     __syncthreads();
     for (int h = threadIdx.x; h < H; h += blockDim.x) {
-        float mx = -INFINITY;
-        for (int w = 0; w < 4; ++w) mx = fmaxf(mx, s_m[w * H + h]);
-        float l = 0.0f;
-        for (int w = 0; w < 4; ++w) l += s_l[w * H + h] > 0.0f ? s_l[w * H + h] * expf(s_m[w * H + h] - mx) : 0.0f;
         float* o = st + (((size_t)m * n_split + split) * H + h) * 2;
-        o[0] = mx;
-        o[1] = l;
+        o[0] = s_m[h];
+        o[1] = s_l[h];
     }
 }
 
@@ -387,7 +499,13 @@ __global__ __launch_bounds__(256) void window_mix_kernel(int H, int G, int D, in
                 const int h = o / V, c = o % V;
                 const float* vbase = cache + (size_t)G * D + (size_t)(h / rep) * V + c;
                 float a = acc[r];
-                for (int jj = 0; jj < nt; ++jj) a = fmaf(s_w[h * kMixTile + jj], vbase[(size_t)s_row[jj] * cstride], a);
+                for (int j0 = 0; j0 < nt; j0 += 8) {  // eight values requested together (keys beyond the tile weigh nothing)
+                    float vv[8];
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) vv[u] = vbase[(size_t)s_row[min(j0 + u, nt - 1)] * cstride];
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) a = fmaf(s_w[h * kMixTile + j0 + u], vv[u], a);
+                }
                 acc[r] = a;
             }
         }
@@ -407,6 +525,7 @@ __global__ __launch_bounds__(256) void window_merge_kernel(const float* po, int 
     const float* base = po + (size_t)m * n_split * H * V;
     for (int p = threadIdx.x; p < H * V / 2; p += blockDim.x) {  // a pair of channels: (2i, 2i + 1) of a head
         float a = 0.0f, b = 0.0f;
+#pragma unroll 8
         for (int s2 = 0; s2 < n_split; ++s2) {
             a += base[(size_t)s2 * H * V + 2 * p];
             b += base[(size_t)s2 * H * V + 2 * p + 1];
@@ -520,100 +639,113 @@ __global__ __launch_bounds__(256) void delta_prep_kernel(float* qk, int ldqk, in
 }
 
 // The recurrence of a head runs column by column of its state: u_c = beta (v_c - S[:, c] . k), S[:, c] += k u_c,
-// o_c = S[:, c] . q touch no other column.  A wave owns kDeltaCols columns, its lanes split the D rows (RPL rows a lane), so both
-// column sums are wave reductions and a token needs no barrier; a workgroup's four waves take neighbouring columns and the
-// grid covers (entry, head, column group): many more waves than heads.  Every wave reads the token's q, k and decay itself (one
-// coalesced load per vector, shared through the caches), one token ahead of its use.
-constexpr int kDeltaCols = 4;
+// o_c = S[:, c] . q touch no other column.  A column sits on the 16 lanes of one DPP row (lane i holds the RPL rows from i RPL
+// on), a wave holds four columns, so the four column sums of a token are ONE row-wise reduction (four DPP adds); a workgroup's
+// four waves take 16 neighbouring columns and the grid covers (entry, head, 16 columns).  The tokens' q, k, decay, values and
+// beta reach the waves through the LDS, kDeltaBlock tokens at a time: the workgroup fetches a block together (few wide loads a
+// thread) while it works on the block before — one barrier per block, none per token.
+constexpr int kDeltaCols = 16;   // columns per workgroup
+constexpr int kDeltaBlock = 8;   // tokens staged together
 template <int RPL>
 __global__ __launch_bounds__(256) void delta_scan_kernel(const float* qk, int ldqk, const float* v, int ldv, const float* beta, int ldb,
                                                          const float* dec, int ldd, float* out, int ldo, int H, int G, int D, int V,
                                                          float* state, size_t slot_stride, const int* ent_start, const int* ent_len,
                                                          const int* ent_slot) {
-    const int e = blockIdx.x, h = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int c0 = (blockIdx.z * 4 + wave) * kDeltaCols;
+    extern __shared__ __attribute__((aligned(16))) float s_delta[];
+    constexpr int Dp = 16 * RPL, TS = 3 * Dp + 20;  // a token's stage: q | k | g (Dp each) | v (16) | beta | pad
+    constexpr int kDeltaFetch = (kDeltaBlock * TS + 255) / 256;  // loads a thread has in flight for a block
+    const int e = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int rl = lane & 15, cl = wave * 4 + (lane >> 4), c = blockIdx.z * kDeltaCols + cl;
     const int n = ent_len[e], m0 = ent_start[e];
-    if (n <= 0 || c0 >= V) return;
+    if (n <= 0) return;
+    const bool col_ok = c < V;
     const int kvh = h / (H / G);
     float* Sg = state + (size_t)ent_slot[e] * slot_stride + (size_t)h * D * V;
-    float S[kDeltaCols][RPL];
+    float S[RPL];
 #pragma unroll
-    for (int c = 0; c < kDeltaCols; ++c)
+    for (int r = 0; r < RPL; ++r) {
+        const int d = rl * RPL + r;
+        S[r] = (d < D && col_ok) ? Sg[(size_t)d * V + c] : 0.0f;
+    }
+    float pre[kDeltaFetch];
+    auto fetch = [&](int t0) {
 #pragma unroll
-        for (int r = 0; r < RPL; ++r) {
-            const int d = lane + 64 * r;
-            S[c][r] = (d < D && c0 + c < V) ? Sg[(size_t)d * V + c0 + c] : 0.0f;
+        for (int i = 0; i < kDeltaFetch; ++i) {
+            const int idx = tid + 256 * i, tt = idx / TS, o = idx % TS;
+            float val = 0.0f;
+            if (tt < kDeltaBlock && t0 + tt < n) {
+                const size_t m = (size_t)(m0 + t0 + tt);
+                if (o < Dp) val = o < D ? qk[m * ldqk + (size_t)kvh * D + o] : 0.0f;
+                else if (o < 2 * Dp) val = o - Dp < D ? qk[m * ldqk + (size_t)(G + kvh) * D + (o - Dp)] : 0.0f;
+                else if (o < 3 * Dp) val = o - 2 * Dp < D ? dec[m * ldd + (size_t)h * D + (o - 2 * Dp)] : 0.0f;
+                else if (o < 3 * Dp + 16) val = blockIdx.z * kDeltaCols + (o - 3 * Dp) < V ? v[m * ldv + (size_t)h * V + blockIdx.z * kDeltaCols + (o - 3 * Dp)] : 0.0f;
+                else if (o == 3 * Dp + 16) val = beta[m * ldb + h];
+            }
+            pre[i] = val;
         }
-    float q[RPL], k[RPL], g[RPL], vv[kDeltaCols], bt;
-    auto fetch = [&](int t, float* fq, float* fk, float* fg, float* fv, float& fb) {
-        const size_t m = (size_t)(m0 + t);
-#pragma unroll
-        for (int r = 0; r < RPL; ++r) {
-            const int d = lane + 64 * r;
-            const bool ok = d < D;
-            fq[r] = ok ? qk[m * ldqk + (size_t)kvh * D + d] : 0.0f;
-            fk[r] = ok ? qk[m * ldqk + (size_t)(G + kvh) * D + d] : 0.0f;
-            fg[r] = ok ? dec[m * ldd + (size_t)h * D + d] : 0.0f;
-        }
-#pragma unroll
-        for (int c = 0; c < kDeltaCols; ++c) fv[c] = c0 + c < V ? v[m * ldv + (size_t)h * V + c0 + c] : 0.0f;
-        fb = beta[m * ldb + h];
     };
-    fetch(0, q, k, g, vv, bt);
-    for (int t = 0; t < n; ++t) {
-        float nq[RPL], nk[RPL], ng[RPL], nv[kDeltaCols], nb = 0.0f;
-        if (t + 1 < n) fetch(t + 1, nq, nk, ng, nv, nb);
-        float part[kDeltaCols];
+    auto stash = [&](int buf) {
 #pragma unroll
-        for (int c = 0; c < kDeltaCols; ++c) {
+        for (int i = 0; i < kDeltaFetch; ++i) {
+            const int idx = tid + 256 * i;
+            if (idx < kDeltaBlock * TS) s_delta[buf * kDeltaBlock * TS + idx] = pre[i];
+        }
+    };
+    fetch(0);
+    stash(0);
+    for (int t0 = 0, blk = 0; t0 < n; t0 += kDeltaBlock, ++blk) {
+        const bool more = t0 + kDeltaBlock < n;
+        if (more) fetch(t0 + kDeltaBlock);
+        __syncthreads();  // this block is staged; the other buffer has been consumed
+        const float* sb = s_delta + (blk & 1) * kDeltaBlock * TS;
+        const int nb = min(kDeltaBlock, n - t0);
+#pragma unroll
+        for (int i = 0; i < kDeltaBlock; ++i) {
+            if (i >= nb) break;
+            const float* st = sb + i * TS;
+            float q[RPL], k[RPL], g[RPL];
+            if constexpr (RPL % 4 == 0) {  // a lane's rows are consecutive: 16-byte LDS reads
+#pragma unroll
+                for (int r = 0; r < RPL; r += 4) {
+                    const f32x4 a4 = *reinterpret_cast<const f32x4*>(st + rl * RPL + r);
+                    const f32x4 b4 = *reinterpret_cast<const f32x4*>(st + Dp + rl * RPL + r);
+                    const f32x4 c4 = *reinterpret_cast<const f32x4*>(st + 2 * Dp + rl * RPL + r);
+                    q[r] = a4.x; q[r + 1] = a4.y; q[r + 2] = a4.z; q[r + 3] = a4.w;
+                    k[r] = b4.x; k[r + 1] = b4.y; k[r + 2] = b4.z; k[r + 3] = b4.w;
+                    g[r] = c4.x; g[r + 1] = c4.y; g[r + 2] = c4.z; g[r + 3] = c4.w;
+                }
+            } else {
+#pragma unroll
+                for (int r = 0; r < RPL; ++r) {
+                    q[r] = st[rl * RPL + r];
+                    k[r] = st[Dp + rl * RPL + r];
+                    g[r] = st[2 * Dp + rl * RPL + r];
+                }
+            }
+            const float vv = st[3 * Dp + cl], bt = st[3 * Dp + 16];
             float a = 0.0f;
 #pragma unroll
             for (int r = 0; r < RPL; ++r) {
-                S[c][r] *= g[r];
-                a = fmaf(S[c][r], k[r], a);
+                S[r] *= g[r];
+                a = fmaf(S[r], k[r], a);
             }
-            part[c] = a;
-        }
-#pragma unroll
-        for (int c = 0; c < kDeltaCols; ++c) part[c] = wave_allsum(part[c]);
-#pragma unroll
-        for (int c = 0; c < kDeltaCols; ++c) {
-            const float u = bt * (vv[c] - part[c]);
-            float a = 0.0f;
+            const float u = bt * (vv - row16_allsum(a));
+            a = 0.0f;
 #pragma unroll
             for (int r = 0; r < RPL; ++r) {
-                S[c][r] = fmaf(k[r], u, S[c][r]);
-                a = fmaf(S[c][r], q[r], a);
+                S[r] = fmaf(k[r], u, S[r]);
+                a = fmaf(S[r], q[r], a);
             }
-            part[c] = a;
+            a = row16_allsum(a);
+            if (rl == 0 && col_ok) out[(size_t)(m0 + t0 + i) * ldo + (size_t)h * V + c] = a;
         }
-#pragma unroll
-        for (int c = 0; c < kDeltaCols; ++c) part[c] = wave_allsum(part[c]);
-        if (lane < kDeltaCols && c0 + lane < V) {
-            float o = part[0];
-#pragma unroll
-            for (int c = 1; c < kDeltaCols; ++c) o = lane == c ? part[c] : o;
-            out[(size_t)(m0 + t) * ldo + (size_t)h * V + c0 + lane] = o;
-        }
-        if (t + 1 < n) {
-#pragma unroll
-            for (int r = 0; r < RPL; ++r) {
-                q[r] = nq[r];
-                k[r] = nk[r];
-                g[r] = ng[r];
-            }
-#pragma unroll
-            for (int c = 0; c < kDeltaCols; ++c) vv[c] = nv[c];
-            bt = nb;
-        }
+        if (more) stash((blk + 1) & 1);
     }
 #pragma unroll
-    for (int c = 0; c < kDeltaCols; ++c)
-#pragma unroll
-        for (int r = 0; r < RPL; ++r) {
-            const int d = lane + 64 * r;
-            if (d < D && c0 + c < V) Sg[(size_t)d * V + c0 + c] = S[c][r];
-        }
+    for (int r = 0; r < RPL; ++r) {
+        const int d = rl * RPL + r;
+        if (d < D && col_ok) Sg[(size_t)d * V + c] = S[r];
+    }
 }
 
 // one wave per (row, head) vector, in place: v / rms(v) * w * sigmoid(gate)
@@ -641,20 +773,31 @@ int launch_add_rows(float* x, const float* y, int M, int W, hipStream_t s) {
     return ZG_OK;
 }
 
-int launch_causal_conv(const ConvArgs& a, int M, int n_entries, const int* row_off, const int* row_slot, const int* ent_start, const int* ent_len,
-                       const int* ent_slot, hipStream_t s) {
+int launch_causal_conv(const ConvArgs& a, int M, int n_entries, bool one_row_each, const int* row_off, const int* row_slot, const int* ent_start,
+                       const int* ent_len, const int* ent_slot, hipStream_t s) {
     if (M <= 0 || a.C <= 0) return ZG_OK;
     ZG_REQUIRE(a.taps >= 1 && a.taps <= kMaxTaps, ZG_ERR_UNSUPPORTED, "convolution: %d taps (1 to %d)", a.taps, kMaxTaps);
     ZG_REQUIRE(a.in != a.out, ZG_ERR_ARG, "convolution: in place");
     const int bx = a.C >= 256 ? 256 : 64;
     causal_conv_kernel<<<dim3(M, (a.C + bx - 1) / bx), bx, 0, s>>>(a.in, a.ld_in, a.out, a.ld_out, a.C, a.taps, a.w, a.bias, a.pre_bias, a.flags, a.tail,
-                                                                 a.slot_stride, row_off, row_slot);
+                                                                 a.slot_stride, row_off, row_slot, one_row_each ? 1 : 0);
     ZG_HIP(hipGetLastError());
-    if (a.taps > 1) {
+    if (a.taps > 1 && !one_row_each) {
         conv_tail_kernel<<<dim3(n_entries, (a.C + bx - 1) / bx), bx, 0, s>>>(a.in, a.ld_in, a.C, a.taps, a.pre_bias, a.tail, a.slot_stride, ent_start,
                                                                            ent_len, ent_slot);
         ZG_HIP(hipGetLastError());
     }
+    return ZG_OK;
+}
+
+int launch_norm_conv_single(float* x, const float* x0, const float* yl, const float* yr, const float* wl, const float* wr, const float* wb,
+                            const float* wn, float eps, int M, int W, int taps, const float* cw, float* tail, size_t slot_stride,
+                            const int* row_slot, float* out, hipStream_t s, bool* taken) {
+    *taken = false;
+    if (M <= 0 || W > 256 * kSingleRegs || taps < 1 || taps > kMaxTaps) return ZG_OK;
+    norm_conv_single_kernel<<<M, 256, 0, s>>>(x, x0, yl, yr, wl, wr, wb, wn, eps, W, taps, cw, tail, slot_stride, row_slot, out);
+    ZG_HIP(hipGetLastError());
+    *taken = true;
     return ZG_OK;
 }
 
@@ -684,7 +827,9 @@ int launch_window_attention(const float* q, int ldq, float* out, int ldo, int M,
 }
 
 size_t window_split_workspace(int rows, int H, int V, int key_capacity, int* n_split_out) {
-    const int n_split = std::max(1, std::min(kWinSplits, (key_capacity + kMixTile - 1) / kMixTile));
+    // steps of few rows: a share of kMixTile keys (many workgroups per row); portions: shares of kScoreTile keys
+    const int share = rows <= kGemvMaxRows ? kMixTile : kScoreTile;
+    const int n_split = std::max(1, std::min(kWinSplits, (key_capacity + share - 1) / share));
     if (n_split_out) *n_split_out = n_split;
     return (size_t)rows * H * key_capacity + (size_t)rows * n_split * H * 2 + (size_t)rows * n_split * H * V;
 }
@@ -700,7 +845,7 @@ int launch_window_attention_split(const float* q, int ldq, float* out, int ldo, 
     int n_split = 1;
     const size_t need = window_split_workspace(M, H, V, key_capacity, &n_split);
     const int rpl = (D + 63) / 64;
-    const size_t lds_a = ((size_t)H * 64 * rpl + 8 * (size_t)H) * sizeof(float);
+    const size_t lds_a = ((size_t)H * 64 * rpl + (size_t)H * kScoreTile + 2 * (size_t)H) * sizeof(float);
     const size_t lds_b = (2 * (size_t)H * kMixTile + (size_t)H * H + 2 * (size_t)H) * sizeof(float);
     if (!ws || need > ws_floats || H > kWinMaxHeads || H % G != 0 || H * V > 256 * kWinAcc || D > 256 || V % 2 != 0 || lds_a > 60 * 1024 ||
         lds_b > 60 * 1024 || M > 65535)
@@ -757,13 +902,18 @@ int launch_delta_scan(const float* qk, int ldqk, const float* v, int ldv, const 
     if (n_entries <= 0) return ZG_OK;
     ZG_REQUIRE(D >= 1 && D <= 256 && V >= 1 && V <= 256 && G >= 1 && H % G == 0, ZG_ERR_UNSUPPORTED,
                "delta rule: %d heads on %d key heads, %d key and %d value channels per head (at most 256 each)", H, G, D, V);
-    const int rpl = (D + 63) / 64;
-    const dim3 grid(n_entries, H, (V + 4 * kDeltaCols - 1) / (4 * kDeltaCols));
+    const int rpl = (D + 15) / 16;
+    const int rp = rpl <= 1 ? 1 : rpl <= 2 ? 2 : rpl <= 4 ? 4 : rpl <= 8 ? 8 : 16;
+    const size_t stage = (size_t)kDeltaBlock * (3 * 16 * rp + 20);
+    const size_t lds = 2 * stage * sizeof(float);
+    const dim3 grid(n_entries, H, (V + kDeltaCols - 1) / kDeltaCols);
 #define ZG_DELTA(R) \
-    delta_scan_kernel<R><<<grid, 256, 0, s>>>(qk, ldqk, v, ldv, beta, ldb, dec, ldd, out, ldo, H, G, D, V, state, slot_stride, ent_start, ent_len, ent_slot)
-    if (rpl <= 1) ZG_DELTA(1);
-    else if (rpl <= 2) ZG_DELTA(2);
-    else ZG_DELTA(4);
+    delta_scan_kernel<R><<<grid, 256, lds, s>>>(qk, ldqk, v, ldv, beta, ldb, dec, ldd, out, ldo, H, G, D, V, state, slot_stride, ent_start, ent_len, ent_slot)
+    if (rp == 1) ZG_DELTA(1);
+    else if (rp == 2) ZG_DELTA(2);
+    else if (rp == 4) ZG_DELTA(4);
+    else if (rp == 8) ZG_DELTA(8);
+    else ZG_DELTA(16);
 #undef ZG_DELTA
     ZG_HIP(hipGetLastError());
     return ZG_OK;
