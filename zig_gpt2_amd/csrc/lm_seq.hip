@@ -99,7 +99,7 @@ __global__ __launch_bounds__(256) void conv_tail_kernel(const float* in, int ld_
 // products of a layer pass in one launch —
 //   [x += x0]   or   [y = yl, or the mean of the two normed branches (yl / rms * wl + yr / rms * wr) / 2;  x += y / rms(y) * (1 + wb)]
 //   h = x / rms(x) * (1 + wn);   out = h + conv(h) over the slot's tail;   the tail moved on by h.
-constexpr int kSingleRegs = 16;
+constexpr int kSingleRegs = 8;
 __global__ __launch_bounds__(256) void norm_conv_single_kernel(float* x, const float* x0, const float* yl, const float* yr, const float* wl,
                                                                const float* wr, const float* wb, const float* wn, float eps, int W, int taps,
                                                                const float* cw, float* tail, size_t slot_stride, const int* row_slot,
@@ -108,20 +108,26 @@ __global__ __launch_bounds__(256) void norm_conv_single_kernel(float* x, const f
     const int m = blockIdx.x, K = taps - 1;
     float* xr = x + (size_t)m * W;
     float* tl = tail + (size_t)row_slot[m] * slot_stride;
-    float xv[kSingleRegs], yv[kSingleRegs];
+    // every operand of the norms is requested before the first sum: one memory round trip
+    float xv[kSingleRegs], yv[kSingleRegs], zv[kSingleRegs], wlv[kSingleRegs], wrv[kSingleRegs], wbv[kSingleRegs], wnv[kSingleRegs], t0v[kSingleRegs];
 #pragma unroll
     for (int j = 0; j < kSingleRegs; ++j) {
         const int i = threadIdx.x + 256 * j;
-        xv[j] = i < W ? xr[i] + (x0 ? x0[(size_t)m * W + i] : 0.0f) : 0.0f;
-        yv[j] = (i < W && yl) ? yl[(size_t)m * W + i] : 0.0f;
+        const bool ok = i < W;
+        xv[j] = ok ? xr[i] + (x0 ? x0[(size_t)m * W + i] : 0.0f) : 0.0f;
+        yv[j] = (ok && yl) ? yl[(size_t)m * W + i] : 0.0f;
+        zv[j] = (ok && yr) ? yr[(size_t)m * W + i] : 0.0f;
+        wlv[j] = (ok && yr) ? wl[i] : 0.0f;
+        wrv[j] = (ok && yr) ? wr[i] : 0.0f;
+        wbv[j] = (ok && yl) ? wb[i] : 0.0f;
+        wnv[j] = ok ? wn[i] : 0.0f;
+        t0v[j] = (ok && K > 0) ? tl[(size_t)(K - 1) * W + i] : 0.0f;  // the newest tail entry
     }
     if (yl) {
         if (yr) {
-            float zv[kSingleRegs], sa = 0.0f, sb = 0.0f;
+            float sa = 0.0f, sb = 0.0f;
 #pragma unroll
             for (int j = 0; j < kSingleRegs; ++j) {
-                const int i = threadIdx.x + 256 * j;
-                zv[j] = i < W ? yr[(size_t)m * W + i] : 0.0f;
                 sa = fmaf(yv[j], yv[j], sa);
                 sb = fmaf(zv[j], zv[j], sb);
             }
@@ -129,10 +135,7 @@ __global__ __launch_bounds__(256) void norm_conv_single_kernel(float* x, const f
             sb = block_allsum(sb, s_red);
             const float ra = 1.0f / sqrtf(sa / (float)W + eps), rb = 1.0f / sqrtf(sb / (float)W + eps);
 #pragma unroll
-            for (int j = 0; j < kSingleRegs; ++j) {
-                const int i = threadIdx.x + 256 * j;
-                yv[j] = i < W ? 0.5f * (yv[j] * ra * wl[i] + zv[j] * rb * wr[i]) : 0.0f;
-            }
+            for (int j = 0; j < kSingleRegs; ++j) yv[j] = 0.5f * (yv[j] * ra * wlv[j] + zv[j] * rb * wrv[j]);
         }
         float sy = 0.0f;
 #pragma unroll
@@ -140,10 +143,7 @@ __global__ __launch_bounds__(256) void norm_conv_single_kernel(float* x, const f
         sy = block_allsum(sy, s_red);
         const float ry = 1.0f / sqrtf(sy / (float)W + eps);
 #pragma unroll
-        for (int j = 0; j < kSingleRegs; ++j) {
-            const int i = threadIdx.x + 256 * j;
-            if (i < W) xv[j] += yv[j] * ry * (1.0f + wb[i]);
-        }
+        for (int j = 0; j < kSingleRegs; ++j) xv[j] += yv[j] * ry * (1.0f + wbv[j]);
     }
     float sx = 0.0f;
 #pragma unroll
@@ -155,10 +155,10 @@ __global__ __launch_bounds__(256) void norm_conv_single_kernel(float* x, const f
         const int i = threadIdx.x + 256 * j;
         if (i < W) {
             if (x0 || yl) xr[i] = xv[j];
-            const float h = xv[j] * rx * (1.0f + wn[i]);
+            const float h = xv[j] * rx * (1.0f + wnv[j]);
             float acc = cw[(size_t)i * taps + K] * h;
             for (int t = 0; t < K; ++t) {  // tail entry t is taps - 1 - t tokens back; it moves one place towards the front
-                const float tv = tl[(size_t)t * W + i];
+                const float tv = t == K - 1 ? t0v[j] : tl[(size_t)t * W + i];
                 acc = fmaf(cw[(size_t)i * taps + t], tv, acc);
                 if (t > 0) tl[(size_t)(t - 1) * W + i] = tv;
             }
@@ -349,7 +349,7 @@ __device__ __forceinline__ void window_range(int pos, int window, int n_split, i
 }
 
 constexpr int kScoreTile = 128;  // keys whose scores a workgroup holds in the LDS at a time
-constexpr int kScoreKeys = 4;    // keys a wave has in flight
+constexpr int kScoreKeys = 8;    // keys a wave has in flight
 
 template <int RPL>
 __global__ __launch_bounds__(256) void window_scores_kernel(const float* q, int ldq, int H, int G, int D, int V, float scale, int window,
@@ -457,17 +457,17 @@ __global__ __launch_bounds__(256) void window_mix_kernel(int H, int G, int D, in
     const int rep = H / G;
     const size_t cstride = (size_t)G * (D + V);
     for (int i = tid; i < H * H; i += blockDim.x) s_talk[i] = talk ? talk[i] : ((i / H) == (i % H) ? 1.0f : 0.0f);
-    for (int h = tid; h < H; h += blockDim.x) {
-        const float* sp = st + ((size_t)m * n_split * H + h) * 2;
-        float mx = sink ? sink[h] : -INFINITY;
-        for (int s2 = 0; s2 < n_split; ++s2) mx = fmaxf(mx, sp[(size_t)s2 * H * 2]);
-        float z = sink ? expf(sink[h] - mx) : 0.0f;
-        for (int s2 = 0; s2 < n_split; ++s2) {
-            const float l = sp[(size_t)s2 * H * 2 + 1];
-            if (l > 0.0f) z += l * expf(sp[(size_t)s2 * H * 2] - mx);
+    for (int h = tid >> 6; h < H; h += 4) {  // a wave per head, its lanes over the shares (at most kWinSplits = 64): one round trip
+        const int lane = tid & 63;
+        const float* sp = st + (((size_t)m * n_split + lane) * H + h) * 2;
+        const float pm = lane < n_split ? sp[0] : -INFINITY, pl = lane < n_split ? sp[1] : 0.0f;
+        const float sk = sink ? sink[h] : -INFINITY;
+        const float mx = fmaxf(wave_allmax(pm), sk);
+        const float z = wave_allsum(pl > 0.0f ? pl * expf(pm - mx) : 0.0f) + (sink ? expf(sk - mx) : 0.0f);
+        if (lane == 0) {
+            s_M[h] = mx;
+            s_iZ[h] = 1.0f / z;
         }
-        s_M[h] = mx;
-        s_iZ[h] = 1.0f / z;
     }
     float acc[kWinAcc];
 #pragma unroll
@@ -667,22 +667,35 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(const float* qk, int ld
         const int d = rl * RPL + r;
         S[r] = (d < D && col_ok) ? Sg[(size_t)d * V + c] : 0.0f;
     }
+    // what a thread fetches for a block does not change from block to block: source, row stride and token are worked out once
     float pre[kDeltaFetch];
+    const float* src[kDeltaFetch];
+    int stride[kDeltaFetch], tok[kDeltaFetch];
+#pragma unroll
+    for (int i = 0; i < kDeltaFetch; ++i) {
+        const int idx = tid + 256 * i, tt = idx / TS, o = idx % TS;
+        src[i] = qk;
+        stride[i] = 0;
+        tok[i] = -1;
+        if (tt < kDeltaBlock) {
+            const int col = blockIdx.z * kDeltaCols + (o - 3 * Dp);
+            if (o < Dp) {
+                if (o < D) src[i] = qk + (size_t)kvh * D + o, stride[i] = ldqk, tok[i] = tt;
+            } else if (o < 2 * Dp) {
+                if (o - Dp < D) src[i] = qk + (size_t)(G + kvh) * D + (o - Dp), stride[i] = ldqk, tok[i] = tt;
+            } else if (o < 3 * Dp) {
+                if (o - 2 * Dp < D) src[i] = dec + (size_t)h * D + (o - 2 * Dp), stride[i] = ldd, tok[i] = tt;
+            } else if (o < 3 * Dp + 16) {
+                if (col < V) src[i] = v + (size_t)h * V + col, stride[i] = ldv, tok[i] = tt;
+            } else if (o == 3 * Dp + 16) {
+                src[i] = beta + h, stride[i] = ldb, tok[i] = tt;
+            }
+        }
+    }
     auto fetch = [&](int t0) {
 #pragma unroll
-        for (int i = 0; i < kDeltaFetch; ++i) {
-            const int idx = tid + 256 * i, tt = idx / TS, o = idx % TS;
-            float val = 0.0f;
-            if (tt < kDeltaBlock && t0 + tt < n) {
-                const size_t m = (size_t)(m0 + t0 + tt);
-                if (o < Dp) val = o < D ? qk[m * ldqk + (size_t)kvh * D + o] : 0.0f;
-                else if (o < 2 * Dp) val = o - Dp < D ? qk[m * ldqk + (size_t)(G + kvh) * D + (o - Dp)] : 0.0f;
-                else if (o < 3 * Dp) val = o - 2 * Dp < D ? dec[m * ldd + (size_t)h * D + (o - 2 * Dp)] : 0.0f;
-                else if (o < 3 * Dp + 16) val = blockIdx.z * kDeltaCols + (o - 3 * Dp) < V ? v[m * ldv + (size_t)h * V + blockIdx.z * kDeltaCols + (o - 3 * Dp)] : 0.0f;
-                else if (o == 3 * Dp + 16) val = beta[m * ldb + h];
-            }
-            pre[i] = val;
-        }
+        for (int i = 0; i < kDeltaFetch; ++i)
+            pre[i] = (tok[i] >= 0 && t0 + tok[i] < n) ? src[i][(size_t)(m0 + t0 + tok[i]) * stride[i]] : 0.0f;
     };
     auto stash = [&](int buf) {
 #pragma unroll
