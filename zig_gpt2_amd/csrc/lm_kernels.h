@@ -34,7 +34,6 @@ struct Linear {
     int ldc = 0;
     int M = 0, N = 0, K = 0;
     int act = ACT_NONE;
-    const float* bias = nullptr;  // [N], added before the activation (one vector for every batch: not with nz > 1 or groups)
     int a_glu = 0;  // > 0 (row-vector kernel only): A rows are [gate (a_glu) | up (a_glu)] and enter as silu(gate) * up, K = a_glu
     int nz = 1;
     long long a_zoff = 0, b_zoff = 0, c_zoff = 0;

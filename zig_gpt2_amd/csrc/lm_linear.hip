@@ -30,7 +30,6 @@ struct LinArgs {
     const int* a_rows;
     const int* z_group;
     const int* grp_off;
-    const float* bias;
     long long a_zoff, b_zoff, c_zoff;
     int lda, ldb, ldc;
     int M, N, K;
@@ -145,8 +144,8 @@ __global__ __launch_bounds__(256) void lm_gemv_kernel(const LinArgs p) {
     for (int m = 0; m < MR; ++m) {
         const float s0 = wave_allsum(acc0[m]), s1 = wave_allsum(acc1[m]);
         if (lane == 0 && m < p.M) {
-            C[(long long)m * p.ldc + n0] = apply_act(s0 + (p.bias ? p.bias[n0] : 0.0f), p.act);
-            if (two) C[(long long)m * p.ldc + n0 + 1] = apply_act(s1 + (p.bias ? p.bias[n0 + 1] : 0.0f), p.act);
+            C[(long long)m * p.ldc + n0] = apply_act(s0, p.act);
+            if (two) C[(long long)m * p.ldc + n0 + 1] = apply_act(s1, p.act);
         }
     }
 }
@@ -228,7 +227,7 @@ __global__ __launch_bounds__(256) void lm_gemv_ks_kernel(const LinArgs p) {
     if (threadIdx.x < MR * 2) {
         const int m = threadIdx.x >> 1, c = threadIdx.x & 1;
         if (m < p.M && n0 + c < p.N)
-            C[(long long)m * p.ldc + n0 + c] = apply_act((s_part[0][m][c] + s_part[1][m][c]) + (s_part[2][m][c] + s_part[3][m][c]) + (p.bias ? p.bias[n0 + c] : 0.0f), p.act);
+            C[(long long)m * p.ldc + n0 + c] = apply_act((s_part[0][m][c] + s_part[1][m][c]) + (s_part[2][m][c] + s_part[3][m][c]), p.act);
     }
 }
 
@@ -408,7 +407,7 @@ __global__ __launch_bounds__(256) void lm_gemm_kernel(const LinArgs p) {
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
                 const int m = m0 + (wy * WT + i) * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
-                if (m < m_end) C[(long long)m * p.ldc + n] = apply_act(acc[i][j][e] + (p.bias ? p.bias[n] : 0.0f), p.act);
+                if (m < m_end) C[(long long)m * p.ldc + n] = apply_act(acc[i][j][e], p.act);
             }
         }
 }
@@ -421,7 +420,7 @@ int launch_linear(const Linear& L, bool f32, hipStream_t s) {
     ZG_REQUIRE(L.a_div >= 1, ZG_ERR_ARG, "linear: a_div %d", L.a_div);
     LinArgs p;
     p.A = L.A; p.B = L.B; p.C = L.C; p.a_rows = L.a_rows; p.z_group = L.z_group; p.grp_off = L.grp_off;
-    p.bias = L.bias; p.a_zoff = L.a_zoff; p.b_zoff = L.b_zoff; p.c_zoff = L.c_zoff;
+    p.a_zoff = L.a_zoff; p.b_zoff = L.b_zoff; p.c_zoff = L.c_zoff;
     p.lda = L.lda; p.ldb = L.ldb; p.ldc = L.ldc; p.M = L.M; p.N = L.N; p.K = L.K;
     p.a_div = L.a_div; p.act = L.act; p.n_groups = L.grp_off ? L.n_groups : 0; p.a_glu = L.a_glu;
     p.a_vec = ((reinterpret_cast<uintptr_t>(L.A) & 15) == 0 && L.lda % 4 == 0 && L.a_zoff % 4 == 0) ? 1 : 0;

@@ -100,6 +100,7 @@ __global__ __launch_bounds__(256) void conv_tail_kernel(const float* in, int ld_
 //   [x += x0]   or   [y = yl, or the mean of the two normed branches (yl / rms * wl + yr / rms * wr) / 2;  x += y / rms(y) * (1 + wb)]
 //   h = x / rms(x) * (1 + wn);   out = h + conv(h) over the slot's tail;   the tail moved on by h.
 constexpr int kSingleRegs = 8;
+constexpr int kFastTaps = 4;
 __global__ __launch_bounds__(256) void norm_conv_single_kernel(float* x, const float* x0, const float* yl, const float* yr, const float* wl,
                                                                const float* wr, const float* wb, const float* wn, float eps, int W, int taps,
                                                                const float* cw, float* tail, size_t slot_stride, const int* row_slot,
@@ -122,6 +123,19 @@ __global__ __launch_bounds__(256) void norm_conv_single_kernel(float* x, const f
         wbv[j] = (ok && yl) ? wb[i] : 0.0f;
         wnv[j] = ok ? wn[i] : 0.0f;
         t0v[j] = (ok && K > 0) ? tl[(size_t)(K - 1) * W + i] : 0.0f;  // the newest tail entry
+    }
+    // convolutions of up to kFastTaps taps: their weights and the whole tail travel in the same round trip
+    float cwv[kSingleRegs][kFastTaps], tlv[kSingleRegs][kFastTaps - 1];
+    const bool fast = taps <= kFastTaps;
+    if (fast) {
+#pragma unroll
+        for (int j = 0; j < kSingleRegs; ++j) {
+            const int i = threadIdx.x + 256 * j;
+#pragma unroll
+            for (int t = 0; t < kFastTaps; ++t) cwv[j][t] = (i < W && t < taps) ? cw[(size_t)i * taps + t] : 0.0f;
+#pragma unroll
+            for (int t = 0; t < kFastTaps - 1; ++t) tlv[j][t] = (i < W && t < K) ? tl[(size_t)t * W + i] : 0.0f;
+        }
     }
     if (yl) {
         if (yr) {
@@ -156,6 +170,17 @@ __global__ __launch_bounds__(256) void norm_conv_single_kernel(float* x, const f
         if (i < W) {
             if (x0 || yl) xr[i] = xv[j];
             const float h = xv[j] * rx * (1.0f + wnv[j]);
+            if (fast) {
+                float acc = 0.0f;
+#pragma unroll
+                for (int t = 0; t < kFastTaps; ++t) acc = fmaf(cwv[j][t], t == K ? h : t < kFastTaps - 1 ? tlv[j][t] : 0.0f, acc);
+#pragma unroll
+                for (int t = 1; t < kFastTaps - 1; ++t)
+                    if (t < K) tl[(size_t)(t - 1) * W + i] = tlv[j][t];
+                if (K > 0) tl[(size_t)(K - 1) * W + i] = h;
+                out[(size_t)m * W + i] = h + acc;
+                continue;
+            }
             float acc = cw[(size_t)i * taps + K] * h;
             for (int t = 0; t < K; ++t) {  // tail entry t is taps - 1 - t tokens back; it moves one place towards the front
                 const float tv = t == K - 1 ? t0v[j] : tl[(size_t)t * W + i];
