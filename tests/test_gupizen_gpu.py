@@ -205,6 +205,26 @@ def test_general_window_kernel(monkeypatch):
         m.close()
 
 
+@pytest.mark.parametrize("hook", ["ZGPT2_LM_WINDOW_NO_TILES", "ZGPT2_LM_WINDOW_TILES"])
+def test_both_score_kernels_on_all_steps(monkeypatch, hook):
+    """Prompt portions take their scores from matrix-core tiles of 32 rows x 32 keys, steps of few rows from the wave-per-key
+    kernel; the hooks send every step through one of them (ragged row blocks, windows that start inside a tile, two entries)."""
+    monkeypatch.setenv(hook, "1")
+    cfg = gl.config([gl.parallel_layer(heads=6, kv_heads=2, dim=18, vdim=4, window=41, rot_dims=6), gl.parallel_layer(heads=1, kv_heads=1, dim=5, vdim=2, window=0, rot_dims=4)])
+    w = gl.weights(cfg, seed=23)
+    a, b = gl.tokens(24, 150, cfg["vocab"]), gl.tokens(25, 47, cfg["vocab"])
+    oracle = go.Model(cfg, w)
+    ra, rb = oracle.forward(a)[0], oracle.forward(b)[0]
+    m = make(cfg, w)
+    tl.assert_close(run_whole(m, a), ra, "float32")
+    tl.assert_close(run_cut(m, a, [3, 35, 36, 100] + list(range(140, 150))), ra, "float32")
+    sa, sb = m.open(), m.open()
+    got = m.step([(sa, a[:70], list(range(70))), (sb, b, list(range(47)))])
+    tl.assert_close(got[:70], ra[:70], "float32")
+    tl.assert_close(got[70:], rb, "float32")
+    m.close()
+
+
 def _edge_model(window, n, seed):
     """One parallel layer whose attention is sharp (large score factor, no rotary on the scores' channels beyond two): most
     queries put nearly all their weight on one key.  Returns (cfg, weights, oracle, distance of the heaviest key per head and query)."""

@@ -621,7 +621,7 @@ int enqueue_layers(zg_lm* g, int M, int n_ent, bool capturing, bool single) {
             bool split = false;
             ZG_TRY(launch_window_attention_split(g->proj, NP, g->o, HV, M, H, G, D, Vd, d.scale, d.window, L.sink, L.talk, L.vfreq, d_pos, d_slot,
                                                  g->page_table, g->max_pages, g->P, ps.cache, d.window > 0 ? d.window : g->max_pages * g->P, g->win_ws,
-                                                 g->win_ws_floats, s, &split));
+                                                 g->win_ws_floats, d_estart, d_elen, n_ent, s, &split));
             if (!split)
                 ZG_TRY(launch_window_attention(g->proj, NP, g->o, HV, M, H, G, D, Vd, d.scale, d.window, L.sink, L.talk, L.vfreq, d_pos, d_slot,
                                                g->page_table, g->max_pages, g->P, ps.cache, s));

@@ -158,13 +158,15 @@ int launch_window_attention(const float* q, int ldq, float* out, int ldo, int M,
 // The same with a row's keys split over up to kWinSplits workgroups and the scores kept in a workspace (three launches): what
 // steps of few rows need to fill the chip, and prompt portions to compute every score once.  key_capacity: the most keys a row
 // can see (the window, or the longest sequence).  ws: window_split_workspace(rows, ...) floats.  *taken = false (nothing
-// launched) when the workspace is too small or a size is beyond the kernels' limits.
+// launched) when the workspace is too small or a size is beyond the kernels' limits.  Portions (more than kGemvMaxRows rows, heads
+// of at most 128 channels) take their scores from 32 x 32 tiles on the matrix cores in true fp32 (rows of an entry are consecutive
+// rows with consecutive positions: ent_start / ent_len).
 constexpr int kWinSplits = 64;
 size_t window_split_workspace(int rows, int H, int V, int key_capacity, int* n_split_out);
 int launch_window_attention_split(const float* q, int ldq, float* out, int ldo, int M, int H, int G, int D, int V, float scale, int window,
                                   const float* sink, const float* talk, const float* vfreq, const int* row_pos, const int* row_slot,
                                   const int* page_table, int max_pages, int page_tokens, const float* cache, int key_capacity, float* ws,
-                                  size_t ws_floats, hipStream_t s, bool* taken);
+                                  size_t ws_floats, const int* ent_start, const int* ent_len, int n_entries, hipStream_t s, bool* taken);
 
 // ------------------------------------------------------------------------------------------------ real-gated linear recurrent unit
 // Per entry and channel c: r = sigmoid(gr + br), i = sigmoid(gi + bi), a = exp(-8 r softplus(lam)), S = a S + sqrt(1 - a^2) i u,

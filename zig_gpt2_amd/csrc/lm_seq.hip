@@ -463,6 +463,95 @@ __global__ __launch_bounds__(256) void window_scores_kernel(const float* q, int 
     }
 }
 
+// Prompt portions: the scores of 32 consecutive rows of an entry against tiles of 32 keys on the matrix cores, in true fp32
+// (v_mfma_f32_32x32x2_f32 in both precision modes): a key is read once per 32 rows instead of once per row, and no score needs a
+// cross-lane reduction.  Lane (r, half) of a wave holds the channels half * Dh .. + Dh of query row r and of key r (the order of
+// the channels inside the sum is free), so both operands are contiguous runs of a row.  A wave takes (key tile, key head) units;
+// the row's statistics follow in window_stats_kernel.
+typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+
+__device__ __forceinline__ bool rows_find_block(int id, const int* ent_len, int n_entries, int& e, int& b) {
+    for (e = 0; e < n_entries; ++e) {
+        const int nb = (ent_len[e] + 31) / 32;
+        if (id < nb) {
+            b = id;
+            return true;
+        }
+        id -= nb;
+    }
+    return false;
+}
+
+template <int DH>
+__global__ __launch_bounds__(256) void window_scores_mfma_kernel(const float* q, int ldq, int H, int G, int D, int V, float scale, int window,
+                                                                 const int* ent_start, const int* ent_len, int n_entries, const int* row_pos,
+                                                                 const int* row_slot, const int* page_table, int max_pages, int page_tokens,
+                                                                 const float* cache, float* sc, int NK) {
+    int e, b;
+    if (!rows_find_block(blockIdx.x, ent_len, n_entries, e, b)) return;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 31, kh = lane >> 5;
+    const int m0 = ent_start[e] + 32 * b, nrows = min(32, ent_len[e] - 32 * b);
+    const int pos0 = row_pos[m0], pos_last = pos0 + nrows - 1;
+    const int ka = window > 0 ? max(0, pos0 - window + 1) : 0;
+    const int n_tiles = (pos_last - ka) / 32 + 1, units = n_tiles * G;
+    const int* pages = page_table + (size_t)row_slot[m0] * max_pages;
+    const int rep = H / G, Dh = (D + 1) / 2;
+    const size_t cstride = (size_t)G * (D + V);
+    for (int u = blockIdx.y * 4 + wave; u < units; u += 4 * gridDim.y) {
+        const int tile = u / G, g = u % G;
+        const int j = ka + 32 * tile + r;
+        float kreg[DH];
+        {
+            const int jc = min(j, pos_last);
+            const float* kr = cache + ((size_t)pages[(jc / page_tokens) % max_pages] * page_tokens + jc % page_tokens) * cstride + (size_t)g * D + kh * Dh;
+#pragma unroll
+            for (int t = 0; t < DH; ++t) kreg[t] = (j <= pos_last && t < Dh && kh * Dh + t < D) ? kr[t] : 0.0f;
+        }
+        for (int hh = 0; hh < rep; ++hh) {
+            const int h = g * rep + hh;
+            const float* qr = q + (size_t)(m0 + min(r, nrows - 1)) * ldq + (size_t)h * D + kh * Dh;
+            float qreg[DH];
+#pragma unroll
+            for (int t = 0; t < DH; ++t) qreg[t] = (r < nrows && t < Dh && kh * Dh + t < D) ? qr[t] : 0.0f;
+            f32x16_t acc;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
+#pragma unroll
+            for (int t = 0; t < DH; ++t) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(qreg[t], kreg[t], acc, 0, 0, 0);
+            // accumulator element i: query row 8 (i / 4) + 4 half + i % 4 of the block, key r of the tile
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int qi = 8 * (i >> 2) + 4 * kh + (i & 3);
+                const int pi = pos0 + qi;
+                const int jlo = window > 0 ? max(0, pi - window + 1) : 0;
+                if (qi < nrows && j <= pi && j >= jlo) sc[((size_t)(m0 + qi) * H + h) * NK + (j - jlo)] = acc[i] * scale;
+            }
+        }
+    }
+}
+
+// Per row and head the maximum and the sum of exp of the row's scores (a wave per head, its lanes over the keys), filed as the
+// statistics of share 0; the other shares are marked empty.
+__global__ __launch_bounds__(256) void window_stats_kernel(const float* sc, int NK, int H, int window, int n_split, const int* row_pos, float* st) {
+    const int m = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int pos = row_pos[m];
+    const int n_keys = window > 0 ? min(pos + 1, window) : pos + 1;
+    for (int h = wave; h < H; h += 4) {
+        const float* sr = sc + ((size_t)m * H + h) * NK;
+        float mx = -INFINITY;
+        for (int i = lane; i < n_keys; i += 64) mx = fmaxf(mx, sr[i]);
+        mx = wave_allmax(mx);
+        float l = 0.0f;
+        for (int i = lane; i < n_keys; i += 64) l += expf(sr[i] - mx);
+        l = wave_allsum(l);
+        for (int s2 = lane; s2 < n_split; s2 += 64) {
+            float* o = st + (((size_t)m * n_split + s2) * H + h) * 2;
+            o[0] = s2 == 0 ? mx : -INFINITY;
+            o[1] = s2 == 0 ? l : 0.0f;
+        }
+    }
+}
+
 __global__ __launch_bounds__(256) void window_mix_kernel(int H, int G, int D, int V, int window, const float* sink, const float* talk,
                                                          const int* row_pos, const int* row_slot, const int* page_table, int max_pages,
                                                          int page_tokens, const float* cache, const float* sc, int NK, const float* st,
@@ -875,7 +964,7 @@ size_t window_split_workspace(int rows, int H, int V, int key_capacity, int* n_s
 int launch_window_attention_split(const float* q, int ldq, float* out, int ldo, int M, int H, int G, int D, int V, float scale, int window,
                                   const float* sink, const float* talk, const float* vfreq, const int* row_pos, const int* row_slot,
                                   const int* page_table, int max_pages, int page_tokens, const float* cache, int key_capacity, float* ws,
-                                  size_t ws_floats, hipStream_t s, bool* taken) {
+                                  size_t ws_floats, const int* ent_start, const int* ent_len, int n_entries, hipStream_t s, bool* taken) {
     *taken = false;
     if (M <= 0) return ZG_OK;
     if (const char* e = getenv("ZGPT2_LM_WINDOW_GENERAL"))  // test hook: every step through the general kernel
@@ -892,6 +981,26 @@ int launch_window_attention_split(const float* q, int ldq, float* out, int ldo, 
     float* st = sc + (size_t)M * H * key_capacity;
     float* po = st + (size_t)M * n_split * H * 2;
     const dim3 grid(n_split, M);
+    bool tiles = false;
+    if (const char* e = getenv("ZGPT2_LM_WINDOW_TILES")) tiles = atoi(e) != 0;  // test hook: the tiled scores also for steps of few rows
+    if ((M > kGemvMaxRows || tiles) && D <= 128 && ent_start && getenv("ZGPT2_LM_WINDOW_NO_TILES") == nullptr) {
+        // prompt portions: scores of 32 rows x 32 keys on the matrix cores, then the rows' statistics
+        const int dh = (D + 1) / 2;
+        const int max_tiles = (key_capacity + 31) / 32 + 2;
+        const int ksplit = std::max(1, std::min(16, (max_tiles * G + 7) / 8));
+        const dim3 tg((M + 31) / 32 + n_entries, ksplit);
+#define ZG_WT(R)                                                                                                                                   \
+    window_scores_mfma_kernel<R><<<tg, 256, 0, s>>>(q, ldq, H, G, D, V, scale, window, ent_start, ent_len, n_entries, row_pos, row_slot, page_table, \
+                                                    max_pages, page_tokens, cache, sc, key_capacity)
+        if (dh <= 8) ZG_WT(8);
+        else if (dh <= 16) ZG_WT(16);
+        else if (dh <= 32) ZG_WT(32);
+        else ZG_WT(64);
+#undef ZG_WT
+        ZG_HIP(hipGetLastError());
+        window_stats_kernel<<<M, 256, 0, s>>>(sc, key_capacity, H, window, n_split, row_pos, st);
+        ZG_HIP(hipGetLastError());
+    } else {
 #define ZG_WS(R)                                                                                                                              \
     window_scores_kernel<R><<<grid, 256, lds_a, s>>>(q, ldq, H, G, D, V, scale, window, row_pos, row_slot, page_table, max_pages, page_tokens, cache, \
                                                      sc, key_capacity, st)
@@ -899,7 +1008,8 @@ int launch_window_attention_split(const float* q, int ldq, float* out, int ldo, 
     else if (rpl <= 2) ZG_WS(2);
     else ZG_WS(4);
 #undef ZG_WS
-    ZG_HIP(hipGetLastError());
+        ZG_HIP(hipGetLastError());
+    }
     window_mix_kernel<<<grid, 256, lds_b, s>>>(H, G, D, V, window, sink, talk, row_pos, row_slot, page_table, max_pages, page_tokens, cache, sc,
                                                key_capacity, st, po);
     ZG_HIP(hipGetLastError());
