@@ -210,7 +210,8 @@ def test_both_score_kernels_on_all_steps(monkeypatch, hook):
     """Prompt portions take their scores from matrix-core tiles of 32 rows x 32 keys, steps of few rows from the wave-per-key
     kernel; the hooks send every step through one of them (ragged row blocks, windows that start inside a tile, two entries)."""
     monkeypatch.setenv(hook, "1")
-    cfg = gl.config([gl.parallel_layer(heads=6, kv_heads=2, dim=18, vdim=4, window=41, rot_dims=6), gl.parallel_layer(heads=1, kv_heads=1, dim=5, vdim=2, window=0, rot_dims=4)])
+    cfg = gl.config([gl.parallel_layer(heads=6, kv_heads=2, dim=18, vdim=4, window=41, rot_dims=6), gl.parallel_layer(heads=1, kv_heads=1, dim=5, vdim=2, window=0, rot_dims=4),
+                     gl.parallel_layer(heads=18, kv_heads=6, dim=4, vdim=34, window=9, rot_dims=2)])  # more heads than the tiled value product takes
     w = gl.weights(cfg, seed=23)
     a, b = gl.tokens(24, 150, cfg["vocab"]), gl.tokens(25, 47, cfg["vocab"])
     oracle = go.Model(cfg, w)

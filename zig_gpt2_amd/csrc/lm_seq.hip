@@ -632,6 +632,113 @@ __global__ __launch_bounds__(256) void window_mix_kernel(int H, int G, int D, in
     }
 }
 
+// Prompt portions: normalised weights, their mix over the heads and the weighted value sums for 32 consecutive rows of an entry,
+// the value product on the matrix cores in true fp32.  Per tile of kPvKeys keys: every thread takes (row, key) pairs — the
+// weights of all heads from the scores and the rows' statistics (with the sink), mixed in registers, written to the LDS as
+// [head][row][key]; then a wave owns (head, 32 value channels) units whose accumulators live across the tiles: A = the mixed
+// weights of its head (row x key), B = the values of the head's key head (channel x key, read once per 32 rows).  Shares of
+// the block's key range go to blockIdx.y (the merge adds them), groups of kPvUnits * 4 units to blockIdx.z.
+constexpr int kPvKeys = 16;
+constexpr int kPvUnits = 6;  // (head, channel tile) units a wave accumulates
+constexpr int kPvHeads = 16; // most heads of this form (a pair's weights of all heads sit in registers)
+
+__global__ __launch_bounds__(256) void window_mix_mfma_kernel(int H, int G, int D, int V, int window, const float* sink, const float* talk,
+                                                              const int* ent_start, const int* ent_len, int n_entries, const int* row_pos,
+                                                              const int* row_slot, const int* page_table, int max_pages, int page_tokens,
+                                                              const float* cache, const float* sc, int NK, const float* st, int n_split,
+                                                              float* po) {
+    extern __shared__ __attribute__((aligned(16))) float s_pv[];
+    constexpr int KP = kPvKeys + 1;           // padded key stride
+    float* s_w = s_pv;                        // [H][32][KP] mixed weights of the tile
+    float* s_talk = s_w + H * 32 * KP;        // [H H]
+    float* s_M = s_talk + H * H;              // [32][H]
+    float* s_iZ = s_M + 32 * H;               // [32][H]
+    __shared__ int s_row[kPvKeys];
+    int e, b;
+    if (!rows_find_block(blockIdx.x, ent_len, n_entries, e, b)) return;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, kh = lane >> 5;
+    const int m0 = ent_start[e] + 32 * b, nrows = min(32, ent_len[e] - 32 * b);
+    const int pos0 = row_pos[m0], pos_last = pos0 + nrows - 1;
+    const int ka = window > 0 ? max(0, pos0 - window + 1) : 0;
+    const int n_tiles = (pos_last - ka) / kPvKeys + 1, per = (n_tiles + gridDim.y - 1) / gridDim.y;
+    const int t_lo = min(n_tiles, (int)blockIdx.y * per), t_hi = min(n_tiles, t_lo + per);
+    const int* pages = page_table + (size_t)row_slot[m0] * max_pages;
+    const int rep = H / G, ctiles = (V + 31) / 32, units = H * ctiles;
+    const size_t cstride = (size_t)G * (D + V);
+    for (int i = tid; i < H * H; i += blockDim.x) s_talk[i] = talk ? talk[i] : ((i / H) == (i % H) ? 1.0f : 0.0f);
+    for (int i = tid; i < 32 * H; i += blockDim.x) {  // the rows' maximum and denominator per head, the sink counted once
+        const int row = i / H, h = i % H;
+        float mx = 0.0f, iz = 0.0f;
+        if (row < nrows) {
+            const float* sp = st + (((size_t)(m0 + row) * n_split) * H + h) * 2;
+            const float sk = sink ? sink[h] : -INFINITY;
+            mx = fmaxf(sp[0], sk);
+            iz = 1.0f / (sp[1] * expf(sp[0] - mx) + (sink ? expf(sk - mx) : 0.0f));
+        }
+        s_M[i] = mx;
+        s_iZ[i] = iz;
+    }
+    f32x16_t acc[kPvUnits];
+#pragma unroll
+    for (int u = 0; u < kPvUnits; ++u)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[u][i] = 0.0f;
+    const int u0 = (blockIdx.z * 4 + wave) * kPvUnits;  // this wave's first unit
+    for (int tile = t_lo; tile < t_hi; ++tile) {
+        const int j0 = ka + kPvKeys * tile;
+        __syncthreads();  // the tile before has been consumed (and, the first time, the statistics are staged)
+        if (tid < kPvKeys) {
+            const int jc = min(j0 + tid, pos_last);
+            s_row[tid] = pages[(jc / page_tokens) % max_pages] * page_tokens + jc % page_tokens;
+        }
+        for (int pr = tid; pr < 32 * kPvKeys; pr += blockDim.x) {
+            const int row = pr / kPvKeys, kk = pr % kPvKeys, j = j0 + kk, pi = pos0 + row;
+            const int jlo = window > 0 ? max(0, pi - window + 1) : 0;
+            const bool ok = row < nrows && j <= pi && j >= jlo;
+            float p[kPvHeads];  // (registers: the loops over it are unrolled to the kernel's most heads)
+            const float* sr = sc + (size_t)(m0 + min(row, nrows - 1)) * H * NK + (ok ? j - jlo : 0);
+#pragma unroll
+            for (int g = 0; g < kPvHeads; ++g) p[g] = (ok && g < H) ? expf(sr[(size_t)g * NK] - s_M[row * H + g]) * s_iZ[row * H + g] : 0.0f;
+            for (int h = 0; h < H; ++h) {
+                float wsum = 0.0f;
+#pragma unroll
+                for (int g = 0; g < kPvHeads; ++g) wsum = fmaf(g < H ? s_talk[h * H + g] : 0.0f, p[g], wsum);
+                s_w[(h * 32 + row) * KP + kk] = wsum;
+            }
+        }
+        __syncthreads();
+        float vv[kPvUnits][kPvKeys / 2];  // the values of all the wave's units are requested before the first product
+#pragma unroll
+        for (int u = 0; u < kPvUnits; ++u) {
+            const int unit = min(u0 + u, units - 1), h = unit / ctiles, c = (unit % ctiles) * 32 + r;
+            const float* vcol = cache + (size_t)G * D + (size_t)(h / rep) * V + min(c, V - 1);
+#pragma unroll
+            for (int t = 0; t < kPvKeys / 2; ++t) vv[u][t] = c < V ? vcol[(size_t)s_row[kh * (kPvKeys / 2) + t] * cstride] : 0.0f;
+        }
+#pragma unroll
+        for (int u = 0; u < kPvUnits; ++u) {
+            const int unit = u0 + u;
+            if (unit < units) {
+                const float* wrow = s_w + ((unit / ctiles) * 32 + r) * KP + kh * (kPvKeys / 2);
+#pragma unroll
+                for (int t = 0; t < kPvKeys / 2; ++t) acc[u] = __builtin_amdgcn_mfma_f32_32x32x2f32(wrow[t], vv[u][t], acc[u], 0, 0, 0);
+            }
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < kPvUnits; ++u) {
+        const int unit = u0 + u;
+        if (unit < units) {
+            const int h = unit / ctiles, c = (unit % ctiles) * 32 + r;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int qi = 8 * (i >> 2) + 4 * kh + (i & 3);
+                if (qi < nrows && c < V) po[((size_t)(m0 + qi) * n_split + blockIdx.y) * H * V + (size_t)h * V + c] = acc[u][i];
+            }
+        }
+    }
+}
+
 __global__ __launch_bounds__(256) void window_merge_kernel(const float* po, int n_split, float* out, int ldo, int H, int V, const float* vfreq,
                                                            const int* row_pos) {
     const int m = blockIdx.x;
@@ -954,9 +1061,8 @@ int launch_window_attention(const float* q, int ldq, float* out, int ldo, int M,
 }
 
 size_t window_split_workspace(int rows, int H, int V, int key_capacity, int* n_split_out) {
-    // steps of few rows: a share of kMixTile keys (many workgroups per row); portions: shares of kScoreTile keys
-    const int share = rows <= kGemvMaxRows ? kMixTile : kScoreTile;
-    const int n_split = std::max(1, std::min(kWinSplits, (key_capacity + share - 1) / share));
+    // shares of kMixTile keys: up to kWinSplits of them for steps of few rows (many workgroups per row), up to 16 for portions
+    const int n_split = std::max(1, std::min(rows <= kGemvMaxRows ? kWinSplits : 16, (key_capacity + kMixTile - 1) / kMixTile));
     if (n_split_out) *n_split_out = n_split;
     return (size_t)rows * H * key_capacity + (size_t)rows * n_split * H * 2 + (size_t)rows * n_split * H * V;
 }
@@ -983,7 +1089,8 @@ int launch_window_attention_split(const float* q, int ldq, float* out, int ldo, 
     const dim3 grid(n_split, M);
     bool tiles = false;
     if (const char* e = getenv("ZGPT2_LM_WINDOW_TILES")) tiles = atoi(e) != 0;  // test hook: the tiled scores also for steps of few rows
-    if ((M > kGemvMaxRows || tiles) && D <= 128 && ent_start && getenv("ZGPT2_LM_WINDOW_NO_TILES") == nullptr) {
+    const bool tiled = (M > kGemvMaxRows || tiles) && D <= 128 && ent_start && getenv("ZGPT2_LM_WINDOW_NO_TILES") == nullptr;
+    if (tiled) {
         // prompt portions: scores of 32 rows x 32 keys on the matrix cores, then the rows' statistics
         const int dh = (D + 1) / 2;
         const int max_tiles = (key_capacity + 31) / 32 + 2;
@@ -1010,8 +1117,16 @@ int launch_window_attention_split(const float* q, int ldq, float* out, int ldo, 
 #undef ZG_WS
         ZG_HIP(hipGetLastError());
     }
-    window_mix_kernel<<<grid, 256, lds_b, s>>>(H, G, D, V, window, sink, talk, row_pos, row_slot, page_table, max_pages, page_tokens, cache, sc,
-                                               key_capacity, st, po);
+    const size_t lds_c = ((size_t)H * 32 * (kPvKeys + 1) + (size_t)H * H + 64 * (size_t)H) * sizeof(float);
+    if (tiled && H <= kPvHeads && lds_c <= 60 * 1024) {  // the value product of 32 rows at a time on the matrix cores
+        const int units = H * ((V + 31) / 32);
+        const dim3 pg((M + 31) / 32 + n_entries, n_split, (units + 4 * kPvUnits - 1) / (4 * kPvUnits));
+        window_mix_mfma_kernel<<<pg, 256, lds_c, s>>>(H, G, D, V, window, sink, talk, ent_start, ent_len, n_entries, row_pos, row_slot, page_table,
+                                                      max_pages, page_tokens, cache, sc, key_capacity, st, n_split, po);
+    } else {
+        window_mix_kernel<<<grid, 256, lds_b, s>>>(H, G, D, V, window, sink, talk, row_pos, row_slot, page_table, max_pages, page_tokens, cache, sc,
+                                                   key_capacity, st, po);
+    }
     ZG_HIP(hipGetLastError());
     window_merge_kernel<<<M, 256, 0, s>>>(po, n_split, out, ldo, H, V, vfreq, row_pos);
     ZG_HIP(hipGetLastError());
