@@ -497,6 +497,7 @@ __global__ __launch_bounds__(256) void window_scores_mfma_kernel(const float* q,
     const int* pages = page_table + (size_t)row_slot[m0] * max_pages;
     const int rep = H / G, Dh = (D + 1) / 2;
     const size_t cstride = (size_t)G * (D + V);
+    const bool vec = D % 8 == 0 && V % 4 == 0 && ldq % 4 == 0 && ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(cache)) & 15) == 0;
     for (int u = blockIdx.y * 4 + wave; u < units; u += 4 * gridDim.y) {
         const int tile = u / G, g = u % G;
         const int j = ka + 32 * tile + r;
@@ -504,15 +505,31 @@ __global__ __launch_bounds__(256) void window_scores_mfma_kernel(const float* q,
         {
             const int jc = min(j, pos_last);
             const float* kr = cache + ((size_t)pages[(jc / page_tokens) % max_pages] * page_tokens + jc % page_tokens) * cstride + (size_t)g * D + kh * Dh;
+            if (vec) {  // 16-byte loads: a lane's run of channels starts on a 16-byte boundary and is a multiple of four long
 #pragma unroll
-            for (int t = 0; t < DH; ++t) kreg[t] = (j <= pos_last && t < Dh && kh * Dh + t < D) ? kr[t] : 0.0f;
+                for (int t = 0; t < DH; t += 4) {
+                    const f32x4 x = (j <= pos_last && t < Dh) ? *reinterpret_cast<const f32x4*>(kr + t) : f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+                    kreg[t] = x.x; kreg[t + 1] = x.y; kreg[t + 2] = x.z; kreg[t + 3] = x.w;
+                }
+            } else {
+#pragma unroll
+                for (int t = 0; t < DH; ++t) kreg[t] = (j <= pos_last && t < Dh && kh * Dh + t < D) ? kr[t] : 0.0f;
+            }
         }
         for (int hh = 0; hh < rep; ++hh) {
             const int h = g * rep + hh;
             const float* qr = q + (size_t)(m0 + min(r, nrows - 1)) * ldq + (size_t)h * D + kh * Dh;
             float qreg[DH];
+            if (vec) {
 #pragma unroll
-            for (int t = 0; t < DH; ++t) qreg[t] = (r < nrows && t < Dh && kh * Dh + t < D) ? qr[t] : 0.0f;
+                for (int t = 0; t < DH; t += 4) {
+                    const f32x4 x = (r < nrows && t < Dh) ? *reinterpret_cast<const f32x4*>(qr + t) : f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+                    qreg[t] = x.x; qreg[t + 1] = x.y; qreg[t + 2] = x.z; qreg[t + 3] = x.w;
+                }
+            } else {
+#pragma unroll
+                for (int t = 0; t < DH; ++t) qreg[t] = (r < nrows && t < Dh && kh * Dh + t < D) ? qr[t] : 0.0f;
+            }
             f32x16_t acc;
 #pragma unroll
             for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
@@ -639,7 +656,7 @@ __global__ __launch_bounds__(256) void window_mix_kernel(int H, int G, int D, in
 // weights of its head (row x key), B = the values of the head's key head (channel x key, read once per 32 rows).  Shares of
 // the block's key range go to blockIdx.y (the merge adds them), groups of kPvUnits * 4 units to blockIdx.z.
 constexpr int kPvKeys = 16;
-constexpr int kPvUnits = 6;  // (head, channel tile) units a wave accumulates
+constexpr int kPvUnits = 3;  // (head, channel tile) units a wave accumulates (few: two workgroups share a compute unit and hide each other's loads)
 constexpr int kPvHeads = 16; // most heads of this form (a pair's weights of all heads sit in registers)
 
 __global__ __launch_bounds__(256) void window_mix_mfma_kernel(int H, int G, int D, int V, int window, const float* sink, const float* talk,
